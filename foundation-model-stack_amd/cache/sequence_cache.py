@@ -1,0 +1,239 @@
+"""The cache of a model: a slot per live sequence, keys and values per layer
+in pages, and a fixed-size state area per slot.
+
+* A *slot* stands for one sequence: its length, its pages in every group, its
+  row in every state tensor.  Slots are handed out when a batch starts and
+  given back when a sequence ends; the next batch uses them again.
+* A *group* collects the schedule entries whose mixers need the same kind of
+  storage (same kv heads, head size and window).  Every group has storage and
+  a page pool of its own: a windowed group gives pages back as soon as no
+  later query can see them, a full group keeps them to the end.
+* *State* is per-sequence memory of fixed size that a mixer declares (the
+  reference's example is the convolution and scan state of its SSM mixer,
+  fms/modules/ssm.py:98-139).  It is zeroed when a slot is handed out.
+
+Storage layout of a group, for the kernels (csrc/rope.hip):
+  keys   [entry][page][kv head][token in page][head_dim]
+  values [entry][page][kv head][head_dim][token in page]
+"""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from .pages import PAGE_TOKENS, CacheFull, PagePool, pages_for
+
+
+@dataclasses.dataclass(frozen=True)
+class KVNeed:
+    """What an attention-like mixer asks of the cache."""
+
+    kv_heads: int
+    head_dim: int
+    window: int = 0  # 0: all keys; w > 0: the last w keys
+
+
+@dataclasses.dataclass(frozen=True)
+class StateNeed:
+    """Fixed-size memory per sequence: name -> (shape, dtype name)."""
+
+    tensors: Tuple[Tuple[str, Tuple[int, ...], str], ...]
+
+
+class KVGroup:
+    def __init__(self, need: KVNeed, entries: List[int], n_pages: int):
+        self.need = need
+        self.entries = list(entries)
+        self.pool = PagePool(n_pages)
+        self.keys: Optional[torch.Tensor] = None
+        self.values: Optional[torch.Tensor] = None
+        # slot -> logical page list; -1 marks a page given back because the window has passed it
+        self.pages: Dict[int, List[int]] = {}
+
+    def allocate_storage(self, dtype: torch.dtype, device) -> None:
+        n, K, D = self.pool.n_pages, self.need.kv_heads, self.need.head_dim
+        # zero-filled: the attention kernels multiply masked-out positions by zero
+        self.keys = torch.zeros(len(self.entries), n, K, PAGE_TOKENS, D, dtype=dtype, device=device)
+        self.values = torch.zeros(len(self.entries), n, K, D, PAGE_TOKENS, dtype=dtype, device=device)
+
+    def bytes_per_token(self, itemsize: int) -> int:
+        return 2 * len(self.entries) * self.need.kv_heads * self.need.head_dim * itemsize
+
+
+class SequenceCache:
+    def __init__(
+        self,
+        kv_needs: Sequence[Tuple[int, KVNeed]],
+        state_needs: Sequence[Tuple[int, StateNeed]],
+        max_tokens: int,
+        max_slots: int,
+        max_seq_len: int,
+        dtype: torch.dtype = torch.float32,
+        device=None,
+    ):
+        """kv_needs / state_needs: (schedule entry, need) pairs of the entries that own storage.
+
+        max_tokens: the most tokens live sequences hold at any time, each sequence's count
+        rounded up to a page.  device None keeps the bookkeeping only (no storage).
+        """
+        if max_tokens <= 0 or max_slots <= 0:
+            raise ValueError("a cache needs room for at least one token and one slot")
+        self.max_tokens = pages_for(max_tokens) * PAGE_TOKENS
+        self.max_slots = max_slots
+        self.max_seq_len = max_seq_len
+        self.dtype, self.device = dtype, device
+        n_pages = pages_for(max_tokens)
+
+        self.groups: List[KVGroup] = []
+        self.group_of_entry: Dict[int, Tuple[int, int]] = {}  # entry -> (group index, index inside the group)
+        by_need: Dict[KVNeed, KVGroup] = {}
+        for entry, need in kv_needs:
+            group = by_need.get(need)
+            if group is None:
+                group = by_need[need] = KVGroup(need, [], n_pages)
+                self.groups.append(group)
+            self.group_of_entry[entry] = (self.groups.index(group), len(group.entries))
+            group.entries.append(entry)
+
+        self.state: Dict[int, Dict[str, torch.Tensor]] = {}
+        self._state_needs = list(state_needs)
+
+        self._free_slots: List[int] = list(range(max_slots - 1, -1, -1))
+        self._live: Dict[int, int] = {}  # slot -> length
+        if device is not None:
+            for group in self.groups:
+                group.allocate_storage(dtype, device)
+            for entry, need in self._state_needs:
+                self.state[entry] = {
+                    name: torch.zeros((max_slots, *shape), dtype=getattr(torch, dt), device=device)
+                    for name, shape, dt in need.tensors
+                }
+
+    # ---- slots -----------------------------------------------------------
+    def alloc_slot(self) -> int:
+        if not self._free_slots:
+            raise CacheFull(f"all {self.max_slots} sequence slots are in use")
+        slot = self._free_slots.pop()
+        if slot in self._live:
+            raise AssertionError(f"slot {slot} was free while live")
+        self._live[slot] = 0
+        for group in self.groups:
+            group.pages[slot] = []
+        for tensors in self.state.values():
+            for t in tensors.values():
+                t[slot].zero_()
+        return slot
+
+    def free_slot(self, slot: int) -> None:
+        if slot not in self._live:
+            raise ValueError(f"slot {slot} is not live (freed twice, or never handed out)")
+        for group in self.groups:
+            for page in group.pages.pop(slot):
+                if page >= 0:
+                    group.pool.free(page)
+        del self._live[slot]
+        self._free_slots.append(slot)
+
+    def live_slots(self) -> List[int]:
+        return sorted(self._live)
+
+    def length(self, slot: int) -> int:
+        return self._live[slot]
+
+    @property
+    def n_free_slots(self) -> int:
+        return len(self._free_slots)
+
+    # ---- pages -----------------------------------------------------------
+    def pages_needed(self, slot: int, new_tokens: int) -> int:
+        """Pages the full-length groups would have to take for `new_tokens` more tokens (the most of any group)."""
+        new_len = self._live[slot] + new_tokens
+        need = 0
+        for group in self.groups:
+            need = max(need, pages_for(new_len) - len(group.pages[slot]))
+        return max(need, 0)
+
+    def extend(self, slot: int, new_tokens: int) -> int:
+        """Make room for `new_tokens` more tokens of `slot`; returns the position of the first of them.
+
+        Windowed groups first give back the pages that no query of this step can see.
+        Nothing changes if the room cannot be made.
+        """
+        if slot not in self._live:
+            raise ValueError(f"slot {slot} is not live")
+        start = self._live[slot]
+        new_len = start + new_tokens
+        if new_tokens < 0:
+            raise ValueError("a sequence cannot shrink")
+        if new_len > self.max_seq_len:
+            raise IndexError(f"sequence of {new_len} tokens exceeds the model's {self.max_seq_len} positions")
+        # which pages would be released, and is there room afterwards?
+        plans = []
+        for group in self.groups:
+            pages = group.pages[slot]
+            release = []
+            if group.need.window > 0:
+                first_visible = max(0, start - group.need.window + 1)
+                release = [i for i in range(min(first_visible // PAGE_TOKENS, len(pages))) if pages[i] >= 0]
+            want = pages_for(new_len) - len(pages)
+            if want > group.pool.n_free + len(release):
+                raise CacheFull(
+                    f"no room for {new_tokens} more tokens of slot {slot}: {want} pages needed, "
+                    f"{group.pool.n_free + len(release)} free of {group.pool.n_pages}"
+                )
+            plans.append((group, release, want))
+        for group, release, want in plans:
+            pages = group.pages[slot]
+            for i in release:
+                group.pool.free(pages[i])
+                pages[i] = -1
+            for _ in range(max(want, 0)):
+                pages.append(group.pool.alloc())
+        self._live[slot] = new_len
+        return start
+
+    def block_table(self, group_index: int, slots: Sequence[int], n_columns: Optional[int] = None) -> torch.Tensor:
+        """int32 [len(slots), n_columns] page numbers on the host (unused entries and released pages: -1)."""
+        group = self.groups[group_index]
+        width = max([len(group.pages[s]) for s in slots] + [1])
+        if n_columns is not None:
+            if n_columns < width:
+                raise ValueError("block table narrower than the longest sequence")
+            width = n_columns
+        table = torch.full((len(slots), width), -1, dtype=torch.int32)
+        for row, slot in enumerate(slots):
+            pages = group.pages[slot]
+            if pages:
+                table[row, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        return table
+
+    # ---- storage views -----------------------------------------------------
+    def kv_of_entry(self, entry: int) -> Tuple[int, torch.Tensor, torch.Tensor]:
+        """(group index, keys [pages, K, 64, D], values [pages, K, D, 64]) of a schedule entry."""
+        g, i = self.group_of_entry[entry]
+        group = self.groups[g]
+        return g, group.keys[i], group.values[i]
+
+    def state_of_entry(self, entry: int) -> Dict[str, torch.Tensor]:
+        return self.state.get(entry, {})
+
+    def check(self) -> None:
+        """Raise if a slot or a page is lost, held twice or free twice."""
+        if len(set(self._free_slots)) != len(self._free_slots):
+            raise AssertionError("a slot is free twice")
+        if set(self._free_slots) & set(self._live):
+            raise AssertionError("a slot is both free and live")
+        if len(self._free_slots) + len(self._live) != self.max_slots:
+            raise AssertionError("a slot is lost")
+        for group in self.groups:
+            group.pool.check()
+            held = [p for pages in group.pages.values() for p in pages if p >= 0]
+            if len(held) != len(set(held)):
+                raise AssertionError("a page belongs to two sequences")
+            if len(held) != group.pool.n_held:
+                raise AssertionError("pages held by sequences and by the pool differ")
+            if set(group.pages) != set(self._live):
+                raise AssertionError("page lists and live slots differ")

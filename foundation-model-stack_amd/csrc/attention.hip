@@ -1,0 +1,541 @@
+// Causal attention over the paged cache, with grouped kv heads and an
+// optional sliding window.
+//
+//   * attn_generic_kernel: any element type (float32 here), any even head
+//     size up to 256, plain FMA arithmetic.  It is the true 32-bit path.
+//   * attn_prefill_bf16_kernel / attn_decode_bf16_kernel (+ merge): bfloat16
+//     storage, float32 softmax and accumulation, MFMA 16x16x32.
+//
+// The MFMA kernels compute S^T = K Q^T (rows: keys, columns: queries) so that
+// the probabilities come out of the accumulator already in the operand layout
+// of the second product O^T = V^T P^T; no round trip through LDS is needed.
+// Cache layout: see rope.hip.
+#include "common.h"
+#include "fmsamd.h"
+
+// ==========================================================================
+// generic kernel: one block per (head, token)
+// ==========================================================================
+#define GEN_THREADS 256
+
+template <typename T>
+__global__ void __launch_bounds__(GEN_THREADS)
+    attn_generic_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
+                        const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                        const int* __restrict__ block_table, int table_stride, const T* __restrict__ k_cache,
+                        const T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale, int window) {
+  __shared__ float qs[256];
+  __shared__ float ps[GEN_THREADS];
+  __shared__ float scratch[17];
+  const int h = blockIdx.x;
+  const int t = blockIdx.y;
+  const int seq = seq_of_token[t];
+  T* o = out + (size_t)t * out_stride + (size_t)h * head_dim;
+  if (seq < 0) {
+    for (int d = threadIdx.x; d < head_dim; d += blockDim.x) o[d] = from_f32<T>(0.f);
+    return;
+  }
+  const int pos = positions[t];
+  const int lo = window > 0 ? (pos - window + 1 > 0 ? pos - window + 1 : 0) : 0;
+  const int kh = h / (nheads / kvheads);
+  const int* bt = block_table + (size_t)seq * table_stride;
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  const T* qrow = q + (size_t)t * q_stride + (size_t)h * head_dim;
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) qs[d] = to_f32(qrow[d]);
+  __syncthreads();
+
+  float m_run = -1e30f, l_run = 0.f, acc = 0.f;  // acc: this thread's output element d = threadIdx.x
+  for (int base = lo; base <= pos; base += GEN_THREADS) {
+    const int j = base + threadIdx.x;
+    float s = -INFINITY;
+    if (j <= pos) {
+      const T* krow = k_cache + (size_t)bt[j / PAGE_TOKENS] * page_elems +
+                      ((size_t)kh * PAGE_TOKENS + j % PAGE_TOKENS) * head_dim;
+      float dot = 0.f;
+      for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_f32(krow[d]), dot);
+      s = dot * scale;
+    }
+    const float m_new = fmaxf(m_run, block_max(s, scratch));
+    const float p = j <= pos ? expf(s - m_new) : 0.f;
+    const float alpha = expf(m_run - m_new);
+    ps[threadIdx.x] = p;
+    const float psum = block_sum(p, scratch);  // has the barriers that publish ps
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (threadIdx.x < head_dim) {
+      const int d = threadIdx.x;
+      float a = acc * alpha;
+      const int n = pos - base + 1 < GEN_THREADS ? pos - base + 1 : GEN_THREADS;
+      for (int i = 0; i < n; ++i) {
+        const int jj = base + i;
+        const T* vrow = v_cache + (size_t)bt[jj / PAGE_TOKENS] * page_elems +
+                        ((size_t)kh * head_dim + d) * PAGE_TOKENS + jj % PAGE_TOKENS;
+        a = fmaf(ps[i], to_f32(*vrow), a);
+      }
+      acc = a;
+    }
+    __syncthreads();  // ps is overwritten by the next chunk
+  }
+  if (threadIdx.x < head_dim) o[threadIdx.x] = from_f32<T>(l_run > 0.f ? acc / l_run : 0.f);
+}
+
+// ==========================================================================
+// MFMA core.  One wave owns 16*QT query columns and walks over pages of keys.
+// ==========================================================================
+template <int MAXDT, int QT>
+struct WaveState {
+  f32x4 acc[QT][MAXDT];  // O^T tiles: rows d = dt*16 + (lane/16)*4 + i, column = lane%16
+  float m[QT];           // running maximum of this lane's column (equal in the 4 lanes of a column)
+  float l[QT];           // this lane's share of the running sum of its column
+};
+
+__device__ __forceinline__ bf16x8 load_bf16x8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
+__device__ __forceinline__ bf16x4 load_bf16x4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
+
+// qreg[qt][c]: this lane's 8 query elements d = c*32 + (lane/16)*8 .. +8 of its column (zero when absent).
+// qpos/qlo: visible keys of this lane's column are qlo <= key <= qpos (qpos < 0: no key).
+template <int MAXDT, int QT>
+__device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
+                                                const int (&qpos)[QT], const int (&qlo)[QT], int key_lo, int key_hi,
+                                                int page_first, int page_step, const int* __restrict__ bt,
+                                                const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+                                                size_t page_elems, int kh, int head_dim, float scale) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int ndt = head_dim / 16;
+  const int nchunk = (head_dim + 31) / 32;
+  if (key_hi < key_lo) return;
+  const int page_last = key_hi / PAGE_TOKENS;
+  for (int pi = page_first; pi <= page_last; pi += page_step) {
+    const size_t phys = (size_t)bt[pi];
+    const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
+    const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const int key0 = pi * PAGE_TOKENS + half * 32;
+      if (key0 > key_hi || key0 + 31 < key_lo) continue;  // uniform over the wave
+      f32x4 sa[QT], sb[QT];
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        sa[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+        sb[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+#pragma unroll
+      for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
+        if (c < nchunk) {
+          const int d = c * 32 + g * 8;
+          bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0}, kb = {0, 0, 0, 0, 0, 0, 0, 0};
+          if (d < head_dim) {
+            ka = load_bf16x8(kp + (size_t)(half * 32 + r) * head_dim + d);
+            kb = load_bf16x8(kp + (size_t)(half * 32 + 16 + r) * head_dim + d);
+          }
+#pragma unroll
+          for (int qt = 0; qt < QT; ++qt) {
+            sa[qt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[qt][c], sa[qt], 0, 0, 0);
+            sb[qt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[qt][c], sb[qt], 0, 0, 0);
+          }
+        }
+      }
+      bf16x8 pmat[QT];
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const int ja = key0 + g * 4 + i;
+          const int jb = ja + 16;
+          sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale : -INFINITY;
+          sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale : -INFINITY;
+          mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+        const float m_new = fmaxf(st.m[qt], mx);
+        const float alpha = __expf(st.m[qt] - m_new);
+        st.m[qt] = m_new;
+        float psum = 0.f;
+        float pa[4], pb[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          pa[i] = __expf(sa[qt][i] - m_new);
+          pb[i] = __expf(sb[qt][i] - m_new);
+          psum += pa[i] + pb[i];
+        }
+        st.l[qt] = st.l[qt] * alpha + psum;
+        pmat[qt] = bf16x8{(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3],
+                          (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
+#pragma unroll
+        for (int dt = 0; dt < MAXDT; ++dt)
+          if (dt < ndt) st.acc[qt][dt] *= alpha;
+      }
+#pragma unroll
+      for (int dt = 0; dt < MAXDT; ++dt) {
+        if (dt < ndt) {
+          const bf16* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + half * 32 + g * 4;
+          const bf16x4 va = load_bf16x4(vrow);
+          const bf16x4 vb = load_bf16x4(vrow + 16);
+          const bf16x8 v = {va[0], va[1], va[2], va[3], vb[0], vb[1], vb[2], vb[3]};
+#pragma unroll
+          for (int qt = 0; qt < QT; ++qt)
+            st.acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat[qt], st.acc[qt][dt], 0, 0, 0);
+        }
+      }
+    }
+  }
+}
+
+template <int MAXDT, int QT>
+__device__ __forceinline__ void wave_state_init(WaveState<MAXDT, QT>& st) {
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    st.m[qt] = -1e30f;
+    st.l[qt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt) st.acc[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+}
+
+template <int MAXDT>
+__device__ __forceinline__ void load_query(bf16x8 (&dst)[(MAXDT + 1) / 2], const bf16* row, int head_dim) {
+  const int g = (threadIdx.x & (WAVE - 1)) >> 4;
+#pragma unroll
+  for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
+    const int d = c * 32 + g * 8;
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (row != nullptr && d < head_dim) v = load_bf16x8(row + d);
+    dst[c] = v;
+  }
+}
+
+// ==========================================================================
+// prefill: a block is PREFILL_WAVES waves, each with 16*QT consecutive query
+// tokens of one sequence, for one query head.  Keys come from the cache, so a
+// chunk that continues a cached prefix works the same way.
+// ==========================================================================
+#define PREFILL_WAVES 4
+#define PREFILL_QT 2
+#define PREFILL_QBLOCK (PREFILL_WAVES * PREFILL_QT * 16)
+
+template <int MAXDT>
+__global__ void __launch_bounds__(PREFILL_WAVES* WAVE)
+    attn_prefill_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                             const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
+                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
+                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
+                             int window) {
+  constexpr int QT = PREFILL_QT;
+  const int h = blockIdx.y;
+  const int wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int t_begin = qblock_start[blockIdx.x];
+  const int t_end = t_begin + qblock_len[blockIdx.x];
+  const int t0 = t_begin + wave * QT * 16;
+  if (t0 >= t_end) return;
+  const int seq = seq_of_token[t0];
+  if (seq < 0) return;
+  const int kh = h / (nheads / kvheads);
+  const int* bt = block_table + (size_t)seq * table_stride;
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  bf16x8 qreg[QT][(MAXDT + 1) / 2];
+  int qpos[QT], qlo[QT];
+  int key_hi = -1, key_lo = 0x7fffffff;
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int t = t0 + qt * 16 + r;
+    const bool valid = t < t_end;
+    load_query<MAXDT>(qreg[qt], valid ? q + (size_t)t * q_stride + (size_t)h * head_dim : nullptr, head_dim);
+    qpos[qt] = valid ? positions[t] : -1;
+    qlo[qt] = (valid && window > 0 && qpos[qt] - window + 1 > 0) ? qpos[qt] - window + 1 : 0;
+  }
+  // key range of the wave: tokens of a block are consecutive positions of one sequence
+  {
+    const int t_last = (t0 + QT * 16 < t_end ? t0 + QT * 16 : t_end) - 1;
+    key_hi = positions[t_last];
+    const int first = positions[t0];
+    key_lo = (window > 0 && first - window + 1 > 0) ? first - window + 1 : 0;
+  }
+
+  WaveState<MAXDT, QT> st;
+  wave_state_init(st);
+  attn_wave_pages<MAXDT, QT>(st, qreg, qpos, qlo, key_lo, key_hi, key_lo / PAGE_TOKENS, 1, bt, k_cache, v_cache,
+                             page_elems, kh, head_dim, scale);
+
+  const int ndt = head_dim / 16;
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    float l = st.l[qt];
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
+    const int t = t0 + qt * 16 + r;
+    if (t < t_end) {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      bf16* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+#pragma unroll
+      for (int dt = 0; dt < MAXDT; ++dt) {
+        if (dt < ndt) {
+          const f32x4 a = st.acc[qt][dt];
+          const bf16x4 o = {(bf16)(a[0] * inv), (bf16)(a[1] * inv), (bf16)(a[2] * inv), (bf16)(a[3] * inv)};
+          *reinterpret_cast<bf16x4*>(orow + dt * 16 + g * 4) = o;
+        }
+      }
+    }
+  }
+}
+
+// ==========================================================================
+// decode: one query token per sequence.  Grid (split, kv head x head tile,
+// token).  The 16 columns of a wave are query heads that share the kv head.
+// Each block covers `pages_per_block` pages; its waves take them in turn and
+// merge through LDS; blocks of one token merge in attn_decode_merge_kernel.
+// ==========================================================================
+#define DECODE_WAVES 4
+
+template <int MAXDT>
+__global__ void __launch_bounds__(DECODE_WAVES* WAVE)
+    attn_decode_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+                            float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits,
+                            const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                            const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
+                            const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
+                            int window, int pages_per_block, int tile_cols) {
+  extern __shared__ float lds[];  // [wave][tile_cols columns][head_dim + 2]
+  const int split = blockIdx.x;
+  const int group = nheads / kvheads;
+  const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
+  const int kh = blockIdx.y / tiles_per_kv;
+  const int ht = blockIdx.y % tiles_per_kv;
+  const int t = blockIdx.z;
+  const int wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int seq = seq_of_token[t];
+  const int cols = group - ht * tile_cols < tile_cols ? group - ht * tile_cols : tile_cols;  // query heads here
+  const int head0 = kh * group + ht * tile_cols;
+  if (seq < 0) {
+    if (split == 0)
+      for (int i = threadIdx.x; i < cols * head_dim; i += blockDim.x)
+        out[(size_t)t * out_stride + (size_t)head0 * head_dim + i] = (bf16)0.f;
+    return;
+  }
+  const int pos = positions[t];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first_split = (lo / PAGE_TOKENS) / pages_per_block;
+  const int last_split = (pos / PAGE_TOKENS) / pages_per_block;
+  if (split < first_split || split > last_split) return;
+
+  const int* bt = block_table + (size_t)seq * table_stride;
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  bf16x8 qreg[1][(MAXDT + 1) / 2];
+  load_query<MAXDT>(qreg[0], r < cols ? q + (size_t)t * q_stride + (size_t)(head0 + r) * head_dim : nullptr, head_dim);
+  const int qpos[1] = {pos};
+  const int qlo[1] = {lo};
+
+  // this block's keys, and the pages of this wave among them
+  int key_lo = split * pages_per_block * PAGE_TOKENS;
+  int key_hi = key_lo + pages_per_block * PAGE_TOKENS - 1;
+  if (key_lo < lo) key_lo = lo;
+  if (key_hi > pos) key_hi = pos;
+  const int block_first_page = key_lo / PAGE_TOKENS;
+
+  WaveState<MAXDT, 1> st;
+  wave_state_init(st);
+  attn_wave_pages<MAXDT, 1>(st, qreg, qpos, qlo, key_lo, key_hi, block_first_page + wave, DECODE_WAVES, bt, k_cache,
+                            v_cache, page_elems, kh, head_dim, scale);
+
+  // ---- merge the waves of the block through LDS -------------------------
+  const int ndt = head_dim / 16;
+  const int cstride = head_dim + 2;
+  float l = st.l[0];
+  l += __shfl_xor(l, 16, WAVE);
+  l += __shfl_xor(l, 32, WAVE);
+  if (r < cols) {
+    float* dst = lds + ((size_t)wave * tile_cols + r) * cstride;
+    if (g == 0) {
+      dst[head_dim] = st.m[0];
+      dst[head_dim + 1] = l;
+    }
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt)
+      if (dt < ndt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[dt * 16 + g * 4 + i] = st.acc[0][dt][i];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < cols * head_dim; idx += blockDim.x) {
+    const int c = idx / head_dim;
+    const int d = idx % head_dim;
+    float m = -1e30f;
+#pragma unroll
+    for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, lds[((size_t)w * tile_cols + c) * cstride + head_dim]);
+    float o = 0.f, lsum = 0.f;
+#pragma unroll
+    for (int w = 0; w < DECODE_WAVES; ++w) {
+      const float* src = lds + ((size_t)w * tile_cols + c) * cstride;
+      const float f = __expf(src[head_dim] - m);
+      o += f * src[d];
+      lsum += f * src[head_dim + 1];
+    }
+    const int head = head0 + c;
+    if (n_splits == 1) {
+      out[(size_t)t * out_stride + (size_t)head * head_dim + d] = (bf16)(lsum > 0.f ? o / lsum : 0.f);
+    } else {
+      const size_t base = ((size_t)t * nheads + head) * n_splits + split;
+      part_o[base * head_dim + d] = o;
+      if (d == 0) {
+        part_ml[base * 2] = m;
+        part_ml[base * 2 + 1] = lsum;
+      }
+    }
+  }
+}
+
+// one block per (head, token): combine the partial results of the splits
+__global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                         bf16* __restrict__ out, long out_stride, const int* __restrict__ positions,
+                                         const int* __restrict__ seq_of_token, int nheads, int head_dim, int n_splits,
+                                         int window, int pages_per_block) {
+  const int h = blockIdx.x;
+  const int t = blockIdx.y;
+  if (seq_of_token[t] < 0) return;  // the decode kernel wrote zeros
+  const int pos = positions[t];
+  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int first_split = (lo / PAGE_TOKENS) / pages_per_block;
+  const int last_split = (pos / PAGE_TOKENS) / pages_per_block;
+  const size_t base = ((size_t)t * nheads + h) * n_splits;
+  float m = -1e30f;
+  for (int s = first_split; s <= last_split; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float o = 0.f, l = 0.f;
+    for (int s = first_split; s <= last_split; ++s) {
+      const float f = __expf(part_ml[(base + s) * 2] - m);
+      o += f * part_o[(base + s) * head_dim + d];
+      l += f * part_ml[(base + s) * 2 + 1];
+    }
+    out[(size_t)t * out_stride + (size_t)h * head_dim + d] = (bf16)(l > 0.f ? o / l : 0.f);
+  }
+}
+
+// ==========================================================================
+// host entry points
+// ==========================================================================
+static int check_common(const char* name, int n_tokens, int nheads, int kvheads, int head_dim, long q_stride,
+                        long out_stride) {
+  FMS_REQUIRE(n_tokens > 0 && nheads > 0 && kvheads > 0, "%s: bad sizes", name);
+  FMS_REQUIRE(nheads % kvheads == 0, "%s: %d query heads are no multiple of %d kv heads", name, nheads, kvheads);
+  FMS_REQUIRE(head_dim > 0 && head_dim <= 256, "%s: head size %d is outside 1..256", name, head_dim);
+  FMS_REQUIRE(q_stride >= (long)nheads * head_dim && out_stride >= (long)nheads * head_dim,
+              "%s: row strides are smaller than heads x head size", name);
+  return 0;
+}
+
+extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride, int dtype,
+                                   const int* positions, const int* seq_of_token, const int* block_table,
+                                   int table_stride, const void* k_cache, const void* v_cache, int n_tokens,
+                                   int nheads, int kvheads, int head_dim, float scale, int window,
+                                   hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (check_common("attn_generic", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
+  FMS_REQUIRE(n_tokens <= 65535, "attn_generic: %d tokens exceed one launch (65535)", n_tokens);
+  dim3 grid(nheads, n_tokens);
+  if (dtype == FMS_F32)
+    attn_generic_kernel<float><<<grid, GEN_THREADS, 0, stream>>>(
+        (const float*)q, q_stride, (float*)out, out_stride, positions, seq_of_token, block_table, table_stride,
+        (const float*)k_cache, (const float*)v_cache, nheads, kvheads, head_dim, scale, window);
+  else if (dtype == FMS_BF16)
+    attn_generic_kernel<bf16><<<grid, GEN_THREADS, 0, stream>>>(
+        (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, block_table, table_stride,
+        (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window);
+  else
+    FMS_REQUIRE(false, "attn_generic: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("attn_generic");
+  return 0;
+}
+
+extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_stride,
+                                        const int* positions, const int* seq_of_token, const int* qblock_start,
+                                        const int* qblock_len, int n_qblocks, const int* block_table, int table_stride,
+                                        const void* k_cache, const void* v_cache, int n_tokens, int nheads,
+                                        int kvheads, int head_dim, float scale, int window, hipStream_t stream) {
+  if (n_tokens == 0 || n_qblocks == 0) return 0;
+  if (check_common("attn_prefill_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
+  FMS_REQUIRE(head_dim % 16 == 0, "attn_prefill_bf16: head size %d is no multiple of 16", head_dim);
+  FMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attn_prefill_bf16: row strides must keep 16-byte alignment");
+  FMS_REQUIRE(nheads <= 65535, "attn_prefill_bf16: too many heads");
+  dim3 grid(n_qblocks, nheads);
+  dim3 block(PREFILL_WAVES * WAVE);
+#define FMS_PF(M)                                                                                                   \
+  attn_prefill_bf16_kernel<M><<<grid, block, 0, stream>>>(                                                          \
+      (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,          \
+      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window)
+  if (head_dim <= 64)
+    FMS_PF(4);
+  else if (head_dim <= 128)
+    FMS_PF(8);
+  else
+    FMS_PF(16);
+#undef FMS_PF
+  FMS_LAUNCH_CHECK("attn_prefill_bf16");
+  return 0;
+}
+
+extern "C" int fmsamd_attn_prefill_qblock() { return PREFILL_QBLOCK; }
+
+extern "C" long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits) {
+  if (n_splits <= 1) return 0;
+  return (long)n_tokens * nheads * n_splits * (head_dim + 2) * (long)sizeof(float);
+}
+
+extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_stride, void* workspace,
+                                       long workspace_bytes, const int* positions, const int* seq_of_token,
+                                       const int* block_table, int table_stride, const void* k_cache,
+                                       const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
+                                       float scale, int window, int max_context, int pages_per_block,
+                                       hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
+  FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
+  FMS_REQUIRE(q_stride % 8 == 0, "attn_decode_bf16: query row stride must keep 16-byte alignment");
+  FMS_REQUIRE(pages_per_block > 0 && max_context > 0, "attn_decode_bf16: bad split sizes");
+  FMS_REQUIRE(n_tokens <= 65535, "attn_decode_bf16: %d tokens exceed one launch (65535)", n_tokens);
+  const int n_splits = ceil_div(ceil_div(max_context, PAGE_TOKENS), pages_per_block);
+  const long need = fmsamd_attn_decode_workspace(n_tokens, nheads, head_dim, n_splits);
+  FMS_REQUIRE(workspace_bytes >= need, "attn_decode_bf16: workspace of %ld bytes, %ld needed", workspace_bytes, need);
+  const int group = nheads / kvheads;
+  const int tile_cols = head_dim > 128 ? 8 : 16;  // keeps the merge buffer within 64 KB of LDS
+  const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
+  FMS_REQUIRE((long)kvheads * tiles_per_kv <= 65535, "attn_decode_bf16: too many heads");
+  float* part_o = (float*)workspace;
+  float* part_ml = part_o ? part_o + (size_t)n_tokens * nheads * n_splits * head_dim : nullptr;
+  dim3 grid(n_splits, kvheads * tiles_per_kv, n_tokens);
+  dim3 block(DECODE_WAVES * WAVE);
+  const size_t lds_bytes = (size_t)DECODE_WAVES * tile_cols * (head_dim + 2) * sizeof(float);
+#define FMS_DC(M)                                                                                                    \
+  attn_decode_bf16_kernel<M><<<grid, block, lds_bytes, stream>>>(                                                    \
+      (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
+      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
+      window, pages_per_block, tile_cols)
+  if (head_dim <= 64)
+    FMS_DC(4);
+  else if (head_dim <= 128)
+    FMS_DC(8);
+  else
+    FMS_DC(16);
+#undef FMS_DC
+  FMS_LAUNCH_CHECK("attn_decode_bf16");
+  if (n_splits > 1) {
+    dim3 mgrid(nheads, n_tokens);
+    attn_decode_merge_kernel<<<mgrid, 64, 0, stream>>>(part_o, part_ml, (bf16*)out, out_stride, positions,
+                                                       seq_of_token, nheads, head_dim, n_splits, window,
+                                                       pages_per_block);
+    FMS_LAUNCH_CHECK("attn_decode_merge");
+  }
+  return 0;
+}

@@ -1,0 +1,241 @@
+// Embedding gather, residual-add + norm, gated activation, casts and bias adds.
+// All statistics and sums are float32; storage types are template parameters.
+#include <stdarg.h>
+#include <stdio.h>
+
+#include "common.h"
+#include "fmsamd.h"
+
+// --------------------------------------------------------------------------
+// error string
+// --------------------------------------------------------------------------
+static thread_local char g_error[512] = "";
+
+void fmsamd_set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_error, sizeof(g_error), fmt, ap);
+  va_end(ap);
+}
+
+extern "C" const char* fmsamd_last_error() { return g_error; }
+
+extern "C" int fmsamd_abi_version() { return FMSAMD_ABI_VERSION; }
+
+// --------------------------------------------------------------------------
+// embedding: resid[t, :] = float(table[ids[t], :])
+// --------------------------------------------------------------------------
+template <typename TableT>
+__global__ void embed_kernel(const int* __restrict__ ids, const TableT* __restrict__ table, float* __restrict__ out,
+                             int width, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);  // the host has checked the range; never read outside
+  const TableT* row = table + (size_t)id * width;
+  float* o = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) o[i] = to_f32(row[i]);
+}
+
+extern "C" int fmsamd_embed(const int* ids, const void* table, int table_dtype, float* out, int n_tokens, int width,
+                            int vocab, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && width > 0 && vocab > 0, "embed: bad sizes T=%d width=%d vocab=%d", n_tokens, width, vocab);
+  const int threads = width >= 1024 ? 256 : 64;
+  if (table_dtype == FMS_F32)
+    embed_kernel<float><<<n_tokens, threads, 0, stream>>>(ids, (const float*)table, out, width, vocab);
+  else if (table_dtype == FMS_BF16)
+    embed_kernel<bf16><<<n_tokens, threads, 0, stream>>>(ids, (const bf16*)table, out, width, vocab);
+  else
+    FMS_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
+  FMS_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// add + norm.  One block per output row.
+//   s = resid[r] (+ branch[r])            float32 sum, written back to resid
+//   s = s - mean(s)                       if use_mean
+//   y = s * rsqrt(mean(s^2) + eps) (* weight) (+ bias)
+// With `rows`, output row i is computed from stream row rows[i] and the
+// residual is not written back (the stream is not used again).
+// --------------------------------------------------------------------------
+template <typename BranchT, typename WeightT, typename OutT>
+__global__ void add_norm_kernel(float* __restrict__ resid, const BranchT* __restrict__ branch,
+                                const WeightT* __restrict__ weight, const WeightT* __restrict__ bias,
+                                OutT* __restrict__ out, const int* __restrict__ rows, int width, float eps,
+                                int use_mean) {
+  __shared__ float scratch[17];
+  const int r = rows ? rows[blockIdx.x] : blockIdx.x;
+  float* x = resid + (size_t)r * width;
+  const BranchT* b = branch ? branch + (size_t)r * width : nullptr;
+  OutT* o = out + (size_t)blockIdx.x * width;
+
+  constexpr int KEEP = 16;  // values a thread keeps in registers; wider rows are read again
+  float keep[KEEP];
+  float sum = 0.f, sq = 0.f;
+  int n = 0;
+  for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+    float v = x[i];
+    if (b) {
+      v += to_f32(b[i]);
+      if (!rows) x[i] = v;
+    }
+    if (n < KEEP) keep[n] = v;
+    sum += v;
+    sq += v * v;
+  }
+  float mean = 0.f;
+  if (use_mean) {
+    mean = block_sum(sum, scratch) / (float)width;
+    // second moment about the mean, from the kept values
+    sq = 0.f;
+    n = 0;
+    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+      float v = (n < KEEP ? keep[n] : (rows && b ? x[i] + to_f32(b[i]) : x[i])) - mean;
+      sq += v * v;
+    }
+  }
+  const float ms = block_sum(sq, scratch) / (float)width;
+  const float scale = rsqrtf(ms + eps);
+  n = 0;
+  for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+    float v = n < KEEP ? keep[n] : (rows && b ? x[i] + to_f32(b[i]) : x[i]);
+    v = (v - mean) * scale;
+    if (weight) v *= to_f32(weight[i]);
+    if (bias) v += to_f32(bias[i]);
+    o[i] = from_f32<OutT>(v);
+  }
+}
+
+template <typename BranchT, typename WeightT, typename OutT>
+static void launch_add_norm(float* resid, const void* branch, const void* weight, const void* bias, void* out,
+                            const int* rows, int n_out, int width, float eps, int use_mean, hipStream_t stream) {
+  const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  add_norm_kernel<BranchT, WeightT, OutT><<<n_out, threads, 0, stream>>>(
+      resid, (const BranchT*)branch, (const WeightT*)weight, (const WeightT*)bias, (OutT*)out, rows, width, eps,
+      use_mean);
+}
+
+extern "C" int fmsamd_add_norm(float* resid, const void* branch, int act_dtype, const void* weight, const void* bias,
+                               int weight_dtype, void* out, const int* rows, int n_out, int width, float eps,
+                               int use_mean, hipStream_t stream) {
+  if (n_out == 0) return 0;
+  FMS_REQUIRE(n_out > 0 && width > 0, "add_norm: bad sizes rows=%d width=%d", n_out, width);
+  FMS_REQUIRE(eps >= 0.f, "add_norm: eps %g is negative", (double)eps);
+#define FMS_AN(B, W, O)                                                                               \
+  launch_add_norm<B, W, O>(resid, branch, weight, bias, out, rows, n_out, width, eps, use_mean, stream)
+  if (act_dtype == FMS_F32 && weight_dtype == FMS_F32)
+    FMS_AN(float, float, float);
+  else if (act_dtype == FMS_BF16 && weight_dtype == FMS_BF16)
+    FMS_AN(bf16, bf16, bf16);
+  else if (act_dtype == FMS_BF16 && weight_dtype == FMS_F32)
+    FMS_AN(bf16, float, bf16);
+  else if (act_dtype == FMS_F32 && weight_dtype == FMS_BF16)
+    FMS_AN(float, bf16, float);
+  else
+    FMS_REQUIRE(false, "add_norm: unknown dtypes act=%d weight=%d", act_dtype, weight_dtype);
+#undef FMS_AN
+  FMS_LAUNCH_CHECK("add_norm");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// gated activation: out[t, j] = act(gu[t, j] + bg[j]) * (gu[t, hidden + j] + bu[j])
+// --------------------------------------------------------------------------
+__device__ __forceinline__ float activate(float x, int kind) {
+  switch (kind) {
+    case FMS_ACT_SILU:
+      return x / (1.f + expf(-x));
+    case FMS_ACT_GELU:
+      return 0.5f * x * (1.f + erff(x * 0.70710678118654752f));
+    case FMS_ACT_RELU:
+      return fmaxf(x, 0.f);
+    default:
+      return x;
+  }
+}
+
+template <typename T, typename BiasT>
+__global__ void gated_act_kernel(const T* __restrict__ gu, const BiasT* __restrict__ bias, T* __restrict__ out,
+                                 int hidden, int act) {
+  const size_t t = blockIdx.y;
+  const T* g = gu + t * 2 * hidden;
+  const T* u = g + hidden;
+  T* o = out + t * hidden;
+  for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < hidden; j += gridDim.x * blockDim.x) {
+    float gv = to_f32(g[j]), uv = to_f32(u[j]);
+    if (bias) {
+      gv += to_f32(bias[j]);
+      uv += to_f32(bias[hidden + j]);
+    }
+    o[j] = from_f32<T>(activate(gv, act) * uv);
+  }
+}
+
+extern "C" int fmsamd_gated_act(const void* gu, const void* bias, int bias_dtype, void* out, int dtype, int n_tokens,
+                                int hidden, int act, hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && hidden > 0, "gated_act: bad sizes T=%d hidden=%d", n_tokens, hidden);
+  FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gated_act: unknown activation %d", act);
+  FMS_REQUIRE(n_tokens <= 65535, "gated_act: %d tokens exceed one launch (65535)", n_tokens);
+  dim3 grid(ceil_div(hidden, 256) > 64 ? 64 : ceil_div(hidden, 256), n_tokens);
+  if (dtype == FMS_F32 && (bias == nullptr || bias_dtype == FMS_F32))
+    gated_act_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)gu, (const float*)bias, (float*)out, hidden, act);
+  else if (dtype == FMS_BF16 && (bias == nullptr || bias_dtype == FMS_BF16))
+    gated_act_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (const bf16*)bias, (bf16*)out, hidden, act);
+  else if (dtype == FMS_BF16 && bias_dtype == FMS_F32)
+    gated_act_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)gu, (const float*)bias, (bf16*)out, hidden, act);
+  else if (dtype == FMS_F32 && bias_dtype == FMS_BF16)
+    gated_act_kernel<float, bf16><<<grid, 256, 0, stream>>>((const float*)gu, (const bf16*)bias, (float*)out, hidden, act);
+  else
+    FMS_REQUIRE(false, "gated_act: unknown dtypes %d/%d", dtype, bias_dtype);
+  FMS_LAUNCH_CHECK("gated_act");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// cast and bias add
+// --------------------------------------------------------------------------
+template <typename A, typename B>
+__global__ void cast_kernel(const A* __restrict__ in, B* __restrict__ out, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    out[i] = from_f32<B>(to_f32(in[i]));
+}
+
+extern "C" int fmsamd_cast(const void* in, int in_dtype, void* out, int out_dtype, long n, hipStream_t stream) {
+  if (n == 0) return 0;
+  FMS_REQUIRE(n > 0, "cast: negative count");
+  const int blocks = ceil_div(n, 256) > 4096 ? 4096 : ceil_div(n, 256);
+  if (in_dtype == FMS_F32 && out_dtype == FMS_BF16)
+    cast_kernel<float, bf16><<<blocks, 256, 0, stream>>>((const float*)in, (bf16*)out, (size_t)n);
+  else if (in_dtype == FMS_BF16 && out_dtype == FMS_F32)
+    cast_kernel<bf16, float><<<blocks, 256, 0, stream>>>((const bf16*)in, (float*)out, (size_t)n);
+  else
+    FMS_REQUIRE(false, "cast: unsupported %d -> %d", in_dtype, out_dtype);
+  FMS_LAUNCH_CHECK("cast");
+  return 0;
+}
+
+template <typename T, typename BiasT>
+__global__ void bias_add_kernel(T* __restrict__ x, const BiasT* __restrict__ bias, int cols) {
+  T* row = x + (size_t)blockIdx.x * cols;
+  for (int j = threadIdx.x; j < cols; j += blockDim.x) row[j] = from_f32<T>(to_f32(row[j]) + to_f32(bias[j]));
+}
+
+extern "C" int fmsamd_bias_add(void* x, int dtype, const void* bias, int bias_dtype, int rows, int cols,
+                               hipStream_t stream) {
+  if (rows == 0) return 0;
+  FMS_REQUIRE(rows > 0 && cols > 0, "bias_add: bad sizes");
+  if (dtype == FMS_F32 && bias_dtype == FMS_F32)
+    bias_add_kernel<float, float><<<rows, 256, 0, stream>>>((float*)x, (const float*)bias, cols);
+  else if (dtype == FMS_BF16 && bias_dtype == FMS_BF16)
+    bias_add_kernel<bf16, bf16><<<rows, 256, 0, stream>>>((bf16*)x, (const bf16*)bias, cols);
+  else if (dtype == FMS_BF16 && bias_dtype == FMS_F32)
+    bias_add_kernel<bf16, float><<<rows, 256, 0, stream>>>((bf16*)x, (const float*)bias, cols);
+  else if (dtype == FMS_F32 && bias_dtype == FMS_BF16)
+    bias_add_kernel<float, bf16><<<rows, 256, 0, stream>>>((float*)x, (const bf16*)bias, cols);
+  else
+    FMS_REQUIRE(false, "bias_add: unknown dtypes");
+  FMS_LAUNCH_CHECK("bias_add");
+  return 0;
+}

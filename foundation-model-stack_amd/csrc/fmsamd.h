@@ -1,0 +1,93 @@
+// C interface of the gfx950 kernel library.  Every function takes device
+// pointers and a HIP stream, checks its arguments on the host, launches
+// asynchronously, and returns 0 or a negative code; fmsamd_last_error()
+// then holds the reason.  Nothing here allocates device memory.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#define FMSAMD_ABI_VERSION 1
+
+// element types
+#define FMS_F32 0
+#define FMS_BF16 1
+
+// activations of the gated feed-forward
+#define FMS_ACT_SILU 0
+#define FMS_ACT_GELU 1
+#define FMS_ACT_RELU 2
+#define FMS_ACT_IDENTITY 3
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* fmsamd_last_error();
+int fmsamd_abi_version();
+
+// resid[t, :] = float(table[ids[t], :])
+int fmsamd_embed(const int* ids, const void* table, int table_dtype, float* out, int n_tokens, int width, int vocab,
+                 hipStream_t stream);
+
+// resid += branch (float32 sum, written back unless `rows` is given); out = norm(resid) * weight + bias.
+// branch, weight, bias and rows may be null.  act_dtype is the type of branch and out.
+int fmsamd_add_norm(float* resid, const void* branch, int act_dtype, const void* weight, const void* bias,
+                    int weight_dtype, void* out, const int* rows, int n_out, int width, float eps, int use_mean,
+                    hipStream_t stream);
+
+// out[t, j] = act(gu[t, j] + b[j]) * (gu[t, hidden + j] + b[hidden + j])
+int fmsamd_gated_act(const void* gu, const void* bias, int bias_dtype, void* out, int dtype, int n_tokens, int hidden,
+                     int act, hipStream_t stream);
+
+int fmsamd_cast(const void* in, int in_dtype, void* out, int out_dtype, long n, hipStream_t stream);
+int fmsamd_bias_add(void* x, int dtype, const void* bias, int bias_dtype, int rows, int cols, hipStream_t stream);
+
+// cos/sin of position * freqs[i], float32, [max_pos, half]
+int fmsamd_rope_table(const float* freqs, float* cos_t, float* sin_t, int max_pos, int half, hipStream_t stream);
+
+// Rotate the queries of qkv in place; rotate the keys and write keys and values into the paged cache
+// (k_cache/v_cache null: queries only).  cos_t null: no rotation.
+int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* positions, const int* seq_of_token,
+                         const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
+                         int rot_dim, int max_pos, void* k_cache, void* v_cache, int n_tokens, int nheads, int kvheads,
+                         int head_dim, hipStream_t stream);
+
+// causal attention over the cache; any element type, any even head size up to 256
+int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride, int dtype, const int* positions,
+                        const int* seq_of_token, const int* block_table, int table_stride, const void* k_cache,
+                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, float scale,
+                        int window, hipStream_t stream);
+
+// bfloat16 prefill: query blocks of at most fmsamd_attn_prefill_qblock() consecutive tokens of one sequence
+int fmsamd_attn_prefill_qblock();
+int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_stride, const int* positions,
+                             const int* seq_of_token, const int* qblock_start, const int* qblock_len, int n_qblocks,
+                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
+                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
+                             hipStream_t stream);
+
+// bfloat16 decode: one token per sequence, keys split over blocks of `pages_per_block` pages
+long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits);
+int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_stride, void* workspace,
+                            long workspace_bytes, const int* positions, const int* seq_of_token,
+                            const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
+                            int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
+                            int max_context, int pages_per_block, hipStream_t stream);
+
+// c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
+int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,
+                    int K, hipStream_t stream);
+int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const void* bias, int bias_dtype, void* c, int out_dtype,
+                     long ldc, int M, int N, int K, hipStream_t stream);
+int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
+                            int out_dtype, long ldo, int M, int N, int K, hipStream_t stream);
+int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
+                                  int out_dtype, long ldo, int M, int hidden, int K, int act, hipStream_t stream);
+
+// token choice; rng_state is [rows][2] uint64 (seed, counter), advanced by the kernel
+int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature, int top_k,
+                  void* rng_state, int* out_tokens, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

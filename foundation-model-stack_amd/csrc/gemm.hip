@@ -1,0 +1,367 @@
+// Matrix products y = x W^T (+ bias) for weights stored [N, K] with K contiguous,
+// which is how every linear layer of a checkpoint is stored.
+//
+//   * sgemm_nt_kernel: float32 in, float32 FMA accumulation, float32 out.  The
+//     true 32-bit path: no matrix-core shortcut, no reduced-precision inputs.
+//   * gemm_bf16_kernel: bfloat16 in, MFMA 16x16x32 with float32 accumulation,
+//     bfloat16 or float32 out; LDS-tiled 128x128x32.  Any M and N; K % 8 == 0.
+//   * skinny_bf16_kernel: M <= 64 rows of x (decode).  Weight-streaming: a
+//     block owns one or two 16-row tiles of W, its waves split K, operands go
+//     from global memory straight into MFMA registers, partial sums meet in
+//     LDS.  Optional fused gate: out = act(x Wg^T) * (x Wu^T).
+#include "common.h"
+#include "fmsamd.h"
+
+// ==========================================================================
+// float32
+// ==========================================================================
+#define SG_BM 64
+#define SG_BN 64
+#define SG_BK 16
+
+__global__ void __launch_bounds__(256)
+    sgemm_nt_kernel(const float* __restrict__ a, long lda, const float* __restrict__ w, const float* __restrict__ bias,
+                    float* __restrict__ c, long ldc, int M, int N, int K) {
+  __shared__ float as[SG_BK][SG_BM + 1];
+  __shared__ float ws[SG_BK][SG_BN + 1];
+  const int tx = threadIdx.x % 16;  // n direction
+  const int ty = threadIdx.x / 16;  // m direction
+  const int m0 = blockIdx.y * SG_BM;
+  const int n0 = blockIdx.x * SG_BN;
+  float acc[4][4] = {};
+  for (int k0 = 0; k0 < K; k0 += SG_BK) {
+    for (int i = threadIdx.x; i < SG_BM * SG_BK; i += 256) {
+      const int row = i / SG_BK, kk = i % SG_BK;
+      const int m = m0 + row, k = k0 + kk;
+      as[kk][row] = (m < M && k < K) ? a[(size_t)m * lda + k] : 0.f;
+      const int n = n0 + row;
+      ws[kk][row] = (n < N && k < K) ? w[(size_t)n * K + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < SG_BK; ++kk) {
+      float av[4], wv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        av[i] = as[kk][ty * 4 + i];
+        wv[i] = ws[kk][tx * 4 + i];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty * 4 + i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + tx * 4 + j;
+      if (n < N) c[(size_t)m * ldc + n] = acc[i][j] + (bias ? bias[n] : 0.f);
+    }
+  }
+}
+
+extern "C" int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M,
+                               int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  FMS_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_f32: bad sizes M=%d N=%d K=%d", M, N, K);
+  FMS_REQUIRE(lda >= K && ldc >= N, "gemm_f32: leading dimensions too small");
+  dim3 grid(ceil_div(N, SG_BN), ceil_div(M, SG_BM));
+  FMS_REQUIRE(grid.y <= 65535, "gemm_f32: M=%d exceeds one launch", M);
+  sgemm_nt_kernel<<<grid, 256, 0, stream>>>(a, lda, w, bias, c, ldc, M, N, K);
+  FMS_LAUNCH_CHECK("gemm_f32");
+  return 0;
+}
+
+// ==========================================================================
+// bfloat16, any M
+// ==========================================================================
+#define GB_BM 128
+#define GB_BN 128
+#define GB_BK 32
+#define GB_LD 40  // padded LDS row (elements): 80 bytes keeps 16-byte reads conflict-poor
+
+template <typename OutT, typename BiasT>
+__global__ void __launch_bounds__(256)
+    gemm_bf16_kernel(const bf16* __restrict__ a, long lda, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
+                     OutT* __restrict__ c, long ldc, int M, int N, int K) {
+  __shared__ __attribute__((aligned(16))) bf16 as[GB_BM * GB_LD];
+  __shared__ __attribute__((aligned(16))) bf16 ws[GB_BN * GB_LD];
+  const int wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int wm = (wave >> 1) * 64;  // this wave's 64x64 corner inside the block tile
+  const int wn = (wave & 1) * 64;
+  const int m0 = blockIdx.y * GB_BM;
+  const int n0 = blockIdx.x * GB_BN;
+
+  f32x4 acc[4][4];  // [n tile][m tile]: rows n = nt*16 + g*4 + i, column m = mt*16 + r
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  for (int k0 = 0; k0 < K; k0 += GB_BK) {
+    // 128 rows x 4 chunks of 8 elements for each operand; 256 threads take two chunks each
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+      const int idx = threadIdx.x + it * 256;
+      const int row = idx >> 2, ch = idx & 3;
+      const int k = k0 + ch * 8;
+      bf16x8 va = {0, 0, 0, 0, 0, 0, 0, 0}, vw = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (k < K) {
+        if (m0 + row < M) va = *reinterpret_cast<const bf16x8*>(a + (size_t)(m0 + row) * lda + k);
+        if (n0 + row < N) vw = *reinterpret_cast<const bf16x8*>(w + (size_t)(n0 + row) * K + k);
+      }
+      *reinterpret_cast<bf16x8*>(as + row * GB_LD + ch * 8) = va;
+      *reinterpret_cast<bf16x8*>(ws + row * GB_LD + ch * 8) = vw;
+    }
+    __syncthreads();
+    bf16x8 av[4], wv[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      av[t] = *reinterpret_cast<const bf16x8*>(as + (wm + t * 16 + r) * GB_LD + g * 8);
+      wv[t] = *reinterpret_cast<const bf16x8*>(ws + (wn + t * 16 + r) * GB_LD + g * 8);
+    }
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt)
+        acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wv[nt], av[mt], acc[nt][mt], 0, 0, 0);
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int m = m0 + wm + mt * 16 + r;
+    if (m >= M) continue;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int n = n0 + wn + nt * 16 + g * 4 + i;
+        if (n < N) {
+          float v = acc[nt][mt][i];
+          if (bias) v += to_f32(bias[n]);
+          c[(size_t)m * ldc + n] = from_f32<OutT>(v);
+        }
+      }
+    }
+  }
+}
+
+extern "C" int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const void* bias, int bias_dtype, void* c,
+                                int out_dtype, long ldc, int M, int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  FMS_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16: bad sizes M=%d N=%d K=%d", M, N, K);
+  FMS_REQUIRE(K % 8 == 0 && lda % 8 == 0, "gemm_bf16: K=%d and the row stride %ld must be multiples of 8", K, lda);
+  FMS_REQUIRE(lda >= K && ldc >= N, "gemm_bf16: leading dimensions too small");
+  dim3 grid(ceil_div(N, GB_BN), ceil_div(M, GB_BM));
+  FMS_REQUIRE(grid.y <= 65535, "gemm_bf16: M=%d exceeds one launch", M);
+  const bool fb = bias != nullptr && bias_dtype == FMS_F32;
+#define FMS_GB(O, B)                                                                                          \
+  gemm_bf16_kernel<O, B><<<grid, 256, 0, stream>>>((const bf16*)a, lda, (const bf16*)w, (const B*)bias, (O*)c, \
+                                                   ldc, M, N, K)
+  if (out_dtype == FMS_BF16 && !fb)
+    FMS_GB(bf16, bf16);
+  else if (out_dtype == FMS_BF16 && fb)
+    FMS_GB(bf16, float);
+  else if (out_dtype == FMS_F32 && !fb)
+    FMS_GB(float, bf16);
+  else if (out_dtype == FMS_F32 && fb)
+    FMS_GB(float, float);
+  else
+    FMS_REQUIRE(false, "gemm_bf16: unknown output dtype %d", out_dtype);
+#undef FMS_GB
+  FMS_LAUNCH_CHECK("gemm_bf16");
+  return 0;
+}
+
+// ==========================================================================
+// bfloat16, M <= 64
+// ==========================================================================
+
+__device__ __forceinline__ float sk_activate(float x, int kind) {
+  switch (kind) {
+    case FMS_ACT_SILU:
+      return x / (1.f + __expf(-x));
+    case FMS_ACT_GELU:
+      return 0.5f * x * (1.f + erff(x * 0.70710678118654752f));
+    case FMS_ACT_RELU:
+      return fmaxf(x, 0.f);
+    default:
+      return x;
+  }
+}
+
+// NTB: 16-row tiles of W per block (the second tile starts `tile2_offset` rows after the first).
+// MT : 16-row tiles of x.
+// GATED: the second tile is the "up" half; out = act(first) * second, N is the hidden size.
+// SK_WAVES: waves of a block (8, or 4 when NTB*MT > 4 so that the LDS buffer stays under 64 KB).
+template <int SK_WAVES, int NTB, int MT, bool GATED, typename OutT, typename BiasT>
+__global__ void __launch_bounds__(SK_WAVES* WAVE)
+    skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
+                       OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act) {
+  __shared__ float red[SK_WAVES][NTB][MT][16][17];
+  const int wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int n0 = blockIdx.x * 16 * (GATED ? 1 : NTB);
+
+  const bf16* wrow[NTB];
+  bool wok[NTB];
+#pragma unroll
+  for (int t = 0; t < NTB; ++t) {
+    const int n = n0 + (t == 0 ? 0 : (GATED ? tile2_offset : 16 * t)) + r;
+    const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : N;
+    wok[t] = n < limit;
+    wrow[t] = w + (size_t)(wok[t] ? n : 0) * K;
+  }
+  const bf16* xrow[MT];
+  bool xok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    xok[t] = t * 16 + r < M;
+    xrow[t] = x + (size_t)(xok[t] ? t * 16 + r : 0) * ldx;
+  }
+
+  f32x4 acc[NTB][MT];
+#pragma unroll
+  for (int i = 0; i < NTB; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  // K in chunks of 64: lane group g covers k = chunk*64 + g*16 .. +16 (two MFMA steps)
+  const int nchunks = (K + 63) / 64;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int ch = wave; ch < nchunks; ch += SK_WAVES) {
+    const int k = ch * 64 + g * 16;
+    bf16x8 wa[NTB], wb[NTB], xa[MT], xb[MT];
+#pragma unroll
+    for (int t = 0; t < NTB; ++t) {
+      wa[t] = (wok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k) : zero;
+      wb[t] = (wok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k + 8) : zero;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+      xa[t] = (xok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k) : zero;
+      xb[t] = (xok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k + 8) : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < NTB; ++i)
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[i], xa[j], acc[i][j], 0, 0, 0);
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[i], xb[j], acc[i][j], 0, 0, 0);
+      }
+  }
+
+  // partial tiles meet in LDS: red[wave][tile n][tile m][n row][m column]
+#pragma unroll
+  for (int i = 0; i < NTB; ++i)
+#pragma unroll
+    for (int j = 0; j < MT; ++j)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) red[wave][i][j][g * 4 + e][r] = acc[i][j][e];
+  __syncthreads();
+
+  constexpr int OUT_TILES = GATED ? 1 : NTB;
+  for (int idx = threadIdx.x; idx < OUT_TILES * MT * 256; idx += blockDim.x) {
+    const int nn = idx & 15;           // n within tile: fastest, so that stores of a row are contiguous
+    const int mm = (idx >> 4) & 15;    // m within tile
+    const int tj = (idx >> 8) % MT;    // m tile
+    const int ti = (idx >> 8) / MT;    // n tile
+    const int m = tj * 16 + mm;
+    const int n = n0 + ti * 16 + nn;
+    if (m >= M || n >= N) continue;
+    float v = 0.f;
+#pragma unroll
+    for (int wv = 0; wv < SK_WAVES; ++wv) v += red[wv][ti][tj][nn][mm];
+    if (GATED) {
+      float u = 0.f;
+#pragma unroll
+      for (int wv = 0; wv < SK_WAVES; ++wv) u += red[wv][1][tj][nn][mm];
+      if (bias) {
+        v += to_f32(bias[n]);
+        u += to_f32(bias[tile2_offset + n]);
+      }
+      v = sk_activate(v, act) * u;
+    } else if (bias) {
+      v += to_f32(bias[n]);
+    }
+    out[(size_t)m * ldo + n] = from_f32<OutT>(v);
+  }
+}
+
+template <int NTB, int MT, bool GATED>
+static void launch_skinny(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
+                          int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int blocks,
+                          hipStream_t stream) {
+  const bool fb = bias != nullptr && bias_dtype == FMS_F32;
+  constexpr int SK_WAVES = NTB * MT > 4 ? 4 : 8;
+#define FMS_SK(O, B)                                                                             \
+  skinny_bf16_kernel<SK_WAVES, NTB, MT, GATED, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(    \
+      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act)
+  if (out_dtype == FMS_BF16) {
+    if (fb)
+      FMS_SK(bf16, float);
+    else
+      FMS_SK(bf16, bf16);
+  } else {
+    if (fb)
+      FMS_SK(float, float);
+    else
+      FMS_SK(float, bf16);
+  }
+#undef FMS_SK
+}
+
+// out[M, N] = x[M, K] w[N, K]^T (+ bias).  M <= 64.
+extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
+                                       void* out, int out_dtype, long ldo, int M, int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  FMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_bf16: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
+  FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
+  FMS_REQUIRE(ldx >= K && ldo >= N, "gemm_skinny_bf16: leading dimensions too small");
+  FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_bf16: unknown output dtype %d", out_dtype);
+  const int mt = ceil_div(M, 16);
+  // two tiles per block when that still leaves every CU several blocks
+  const bool two = N >= 16384;
+  const int blocks = ceil_div(N, two ? 32 : 16);
+#define FMS_LS(NTB, MT) \
+  launch_skinny<NTB, MT, false>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, blocks, stream)
+  if (two) {
+    if (mt == 1) FMS_LS(2, 1); else if (mt == 2) FMS_LS(2, 2); else if (mt == 3) FMS_LS(2, 3); else FMS_LS(2, 4);
+  } else {
+    if (mt == 1) FMS_LS(1, 1); else if (mt == 2) FMS_LS(1, 2); else if (mt == 3) FMS_LS(1, 3); else FMS_LS(1, 4);
+  }
+#undef FMS_LS
+  FMS_LAUNCH_CHECK("gemm_skinny_bf16");
+  return 0;
+}
+
+// out[M, hidden] = act(x Wg^T + bg) * (x Wu^T + bu) with w = [Wg; Wu] stacked, [2*hidden, K].  M <= 64.
+extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias,
+                                             int bias_dtype, void* out, int out_dtype, long ldo, int M, int hidden,
+                                             int K, int act, hipStream_t stream) {
+  if (M == 0 || hidden == 0) return 0;
+  FMS_REQUIRE(M > 0 && M <= 64 && hidden > 0 && K > 0, "gemm_skinny_gated_bf16: bad sizes M=%d hidden=%d K=%d (M <= 64)",
+              M, hidden, K);
+  FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_gated_bf16: K=%d and the row stride %ld must be multiples of 8", K,
+              ldx);
+  FMS_REQUIRE(ldx >= K && ldo >= hidden, "gemm_skinny_gated_bf16: leading dimensions too small");
+  FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_gated_bf16: unknown output dtype %d", out_dtype);
+  FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gemm_skinny_gated_bf16: unknown activation %d", act);
+  const int mt = ceil_div(M, 16);
+  const int blocks = ceil_div(hidden, 16);
+#define FMS_LG(MT) \
+  launch_skinny<2, MT, true>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, blocks, stream)
+  if (mt == 1) FMS_LG(1); else if (mt == 2) FMS_LG(2); else if (mt == 3) FMS_LG(3); else FMS_LG(4);
+#undef FMS_LG
+  FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
+  return 0;
+}

@@ -1,0 +1,115 @@
+// Rotary position encoding: the cos/sin table, and the fused kernel that
+// rotates queries in place and writes rotated keys and the values into the
+// paged cache.
+//
+// Cache layout of one layer (PAGE_TOKENS tokens per page):
+//   keys    [page][kv head][token in page][head_dim]
+//   values  [page][kv head][head_dim][token in page]      (transposed)
+// so that both the score product (contraction over head_dim) and the mixing
+// product (contraction over tokens) read their contraction index contiguously.
+#include "common.h"
+#include "fmsamd.h"
+
+// cos/sin of position * freq, float32: angle = float(p) * f, as the reference
+// builds its table (outer product of positions and frequencies, then cos/sin).
+__global__ void rope_table_kernel(const float* __restrict__ freqs, float* __restrict__ cos_t, float* __restrict__ sin_t,
+                                  int max_pos, int half) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= max_pos * half) return;
+  const int p = idx / half, i = idx % half;
+  const float angle = (float)p * freqs[i];
+  cos_t[idx] = cosf(angle);
+  sin_t[idx] = sinf(angle);
+}
+
+extern "C" int fmsamd_rope_table(const float* freqs, float* cos_t, float* sin_t, int max_pos, int half,
+                                 hipStream_t stream) {
+  FMS_REQUIRE(max_pos > 0 && half > 0, "rope_table: bad sizes max_pos=%d half=%d", max_pos, half);
+  FMS_REQUIRE((long)max_pos * half < (1L << 31), "rope_table: table too large");
+  rope_table_kernel<<<ceil_div((long)max_pos * half, 256), 256, 0, stream>>>(freqs, cos_t, sin_t, max_pos, half);
+  FMS_LAUNCH_CHECK("rope_table");
+  return 0;
+}
+
+// One block per token.  qkv row = [H*D queries | K*D keys | K*D values].
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
+                                     const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
+                                     int table_stride, const float* __restrict__ cos_t,
+                                     const float* __restrict__ sin_t, int rot_dim, int max_pos, T* __restrict__ k_cache,
+                                     T* __restrict__ v_cache, int nheads, int kvheads, int head_dim) {
+  const int t = blockIdx.x;
+  const int seq = seq_of_token[t];
+  if (seq < 0) return;  // padding row of a fixed-size batch
+  int pos = positions[t];
+  const int tpos = pos < max_pos ? pos : max_pos - 1;  // the host has checked; never read outside the table
+  const int half = head_dim / 2;
+  const int rot_half = rot_dim / 2;
+  T* row = qkv + (size_t)t * row_stride;
+
+  long page = 0;
+  int in_page = pos % PAGE_TOKENS;
+  if (k_cache) page = block_table[(size_t)seq * table_stride + pos / PAGE_TOKENS];
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  const int total = (nheads + 2 * kvheads) * half;
+  for (int idx = threadIdx.x; idx < total; idx += blockDim.x) {
+    const int hh = idx / half;
+    const int i = idx % half;
+    T* p = row + (size_t)hh * head_dim + 2 * i;
+    float a = to_f32(p[0]), b = to_f32(p[1]);
+    if (hh < nheads + kvheads) {
+      if (cos_t && i < rot_half) {
+        const float c = cos_t[(size_t)tpos * rot_half + i];
+        const float s = sin_t[(size_t)tpos * rot_half + i];
+        const float ra = c * a - s * b;
+        const float rb = s * a + c * b;
+        a = ra;
+        b = rb;
+      }
+      if (hh < nheads) {
+        p[0] = from_f32<T>(a);
+        p[1] = from_f32<T>(b);
+      } else if (k_cache) {
+        const int kh = hh - nheads;
+        T* dst = k_cache + page * page_elems + ((size_t)kh * PAGE_TOKENS + in_page) * head_dim + 2 * i;
+        dst[0] = from_f32<T>(a);
+        dst[1] = from_f32<T>(b);
+      }
+    } else if (v_cache) {
+      const int kh = hh - nheads - kvheads;
+      T* dst = v_cache + page * page_elems + ((size_t)kh * head_dim + 2 * i) * PAGE_TOKENS + in_page;
+      dst[0] = from_f32<T>(a);
+      dst[PAGE_TOKENS] = from_f32<T>(b);
+    }
+  }
+}
+
+extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* positions,
+                                    const int* seq_of_token, const int* block_table, int table_stride,
+                                    const float* cos_t, const float* sin_t, int rot_dim, int max_pos, void* k_cache,
+                                    void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
+                                    hipStream_t stream) {
+  if (n_tokens == 0) return 0;
+  FMS_REQUIRE(n_tokens > 0 && nheads > 0 && kvheads > 0 && head_dim > 0, "rope_kv_write: bad sizes");
+  FMS_REQUIRE(head_dim % 2 == 0, "rope_kv_write: head size %d is odd", head_dim);
+  FMS_REQUIRE(rot_dim % 2 == 0 && rot_dim >= 0 && rot_dim <= head_dim, "rope_kv_write: rotary size %d does not fit head size %d",
+              rot_dim, head_dim);
+  FMS_REQUIRE(row_stride >= (long)(nheads + 2 * kvheads) * head_dim, "rope_kv_write: row stride too small");
+  FMS_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "rope_kv_write: key and value cache must come together");
+  FMS_REQUIRE(cos_t == nullptr || max_pos > 0, "rope_kv_write: empty table");
+  const int threads = 256;
+  const float* c = rot_dim > 0 ? cos_t : nullptr;
+  if (dtype == FMS_F32)
+    rope_kv_write_kernel<float><<<n_tokens, threads, 0, stream>>>(
+        (float*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
+        (float*)k_cache, (float*)v_cache, nheads, kvheads, head_dim);
+  else if (dtype == FMS_BF16)
+    rope_kv_write_kernel<bf16><<<n_tokens, threads, 0, stream>>>(
+        (bf16*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
+        (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim);
+  else
+    FMS_REQUIRE(false, "rope_kv_write: unknown dtype %d", dtype);
+  FMS_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}

@@ -1,0 +1,113 @@
+"""The index data of one step: which tokens, of which sequences, at which
+positions, reading which pages.  Built on the host, sent to the device in one
+copy, and handed to every part."""
+
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache import PAGE_TOKENS, SequenceCache
+
+
+@dataclasses.dataclass
+class StepBatch:
+    n_tokens: int
+    n_seqs: int
+    slots: List[int]  # cache slot of each sequence of the step
+    q_lens: List[int]  # tokens each sequence brings
+    starts: List[int]  # position of each sequence's first token
+    is_decode: bool  # every sequence brings exactly one token
+    max_context: int  # longest sequence after this step (host value, bounds the decode split)
+    token_ids: torch.Tensor  # int32 [T]
+    positions: torch.Tensor  # int32 [T]
+    seq_of_token: torch.Tensor  # int32 [T], index into the rows of the block tables (-1: padding row)
+    slot_ids: torch.Tensor  # int32 [B], row of each sequence in the state tensors
+    seq_starts: torch.Tensor  # int32 [B + 1], offsets of the sequences in the token arrays
+    block_tables: Dict[int, torch.Tensor]  # group index -> int32 [B, pages]
+    qblock_start: Optional[torch.Tensor] = None  # query blocks of the bfloat16 prefill kernel
+    qblock_len: Optional[torch.Tensor] = None
+    logit_rows: Optional[torch.Tensor] = None  # int32 [n_wanted] token indices whose logits are wanted
+    n_logit_rows: int = 0
+
+
+def build_batch(
+    cache: SequenceCache,
+    slots: Sequence[int],
+    tokens: Sequence[Sequence[int]],
+    starts: Sequence[int],
+    want: Sequence[Sequence[int]],
+    device,
+    qblock: int,
+) -> StepBatch:
+    """Index arrays of a step.  `starts[b]` is what cache.extend(slot, len(tokens[b])) returned."""
+    B = len(slots)
+    q_lens = [len(t) for t in tokens]
+    T = sum(q_lens)
+    flat_ids: List[int] = []
+    positions: List[int] = []
+    seq_of_token: List[int] = []
+    seq_starts = [0]
+    rows: List[int] = []
+    qb_start: List[int] = []
+    qb_len: List[int] = []
+    for b in range(B):
+        base = seq_starts[-1]
+        flat_ids.extend(int(x) for x in tokens[b])
+        positions.extend(range(starts[b], starts[b] + q_lens[b]))
+        seq_of_token.extend([b] * q_lens[b])
+        seq_starts.append(base + q_lens[b])
+        for w in want[b]:
+            if not 0 <= w < q_lens[b]:
+                raise IndexError(f"wanted place {w} is outside the {q_lens[b]} tokens of sequence {b}")
+            rows.append(base + w)
+        for off in range(0, q_lens[b], qblock):
+            qb_start.append(base + off)
+            qb_len.append(min(qblock, q_lens[b] - off))
+    tables = {g: cache.block_table(g, slots) for g in range(len(cache.groups))}
+
+    # one host buffer, one copy
+    parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows, qb_start, qb_len]
+    sizes = [len(p) for p in parts]
+    table_sizes = {g: t.numel() for g, t in tables.items()}
+    total = sum(sizes) + sum(table_sizes.values())
+    host = torch.empty(total, dtype=torch.int32, pin_memory=torch.cuda.is_available())
+    off = 0
+    spans = []
+    for p, n in zip(parts, sizes):
+        if n:
+            host[off : off + n] = torch.tensor(p, dtype=torch.int32)
+        spans.append((off, n))
+        off += n
+    table_spans = {}
+    for g, t in tables.items():
+        host[off : off + t.numel()] = t.reshape(-1)
+        table_spans[g] = (off, t.shape)
+        off += t.numel()
+    dev = host.to(device, non_blocking=True)
+
+    def span(i):
+        o, n = spans[i]
+        return dev[o : o + n]
+
+    return StepBatch(
+        n_tokens=T,
+        n_seqs=B,
+        slots=list(slots),
+        q_lens=q_lens,
+        starts=list(starts),
+        is_decode=all(n == 1 for n in q_lens),
+        max_context=max(s + n for s, n in zip(starts, q_lens)),
+        token_ids=span(0),
+        positions=span(1),
+        seq_of_token=span(2),
+        slot_ids=span(3),
+        seq_starts=span(4),
+        block_tables={g: dev[o : o + shape[0] * shape[1]].view(shape) for g, (o, shape) in table_spans.items()},
+        qblock_start=span(6),
+        qblock_len=span(7),
+        logit_rows=span(5),
+        n_logit_rows=len(rows),
+    )

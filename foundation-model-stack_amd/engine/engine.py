@@ -1,0 +1,93 @@
+"""The step function: one batch of sequences, each bringing its next tokens,
+run as one ragged batch from the cache; logits come back for the wanted places.
+
+A step runs only the tokens it is given.  Sequences are named by their cache
+slots; a sequence's position is its length in the cache, so the same call
+serves whole prompts, single decoded tokens, and anything between.  There is
+no padding: tokens of all sequences are laid end to end.
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Union
+
+import torch
+
+from ..cache import CacheFull, pages_for
+from ..kernels import ops
+from .batch import StepBatch, build_batch
+from .model import DecoderModel
+
+
+class Engine:
+    def __init__(self, model: DecoderModel, max_tokens: Optional[int] = None, max_slots: Optional[int] = None):
+        """max_tokens: the most tokens live sequences hold at a time, each rounded up to a page of 64
+        (default: one sequence of the model's full length).  max_slots: the most live sequences."""
+        if model.device is None:
+            raise RuntimeError("the model has no weights on a device yet (use get_model)")
+        self.model = model
+        self.device = model.device
+        if max_tokens is None:
+            max_tokens = model.spec.max_seq_len
+        if max_slots is None:
+            max_slots = max(1, pages_for(max_tokens))
+        self.cache = model.make_cache(max_tokens, max_slots)
+        self.qblock = ops.prefill_qblock()
+        self.vocab = model.spec.vocab
+
+    # ---- sequences ---------------------------------------------------------
+    def new_sequence(self) -> int:
+        return self.cache.alloc_slot()
+
+    def end_sequence(self, slot: int) -> None:
+        self.cache.free_slot(slot)
+
+    def length(self, slot: int) -> int:
+        return self.cache.length(slot)
+
+    # ---- the step ------------------------------------------------------------
+    def step(
+        self,
+        slots: Sequence[int],
+        tokens: Sequence[Sequence[int]],
+        want: Union[str, Sequence[Sequence[int]]] = "last",
+    ) -> torch.Tensor:
+        """Append `tokens[b]` to sequence `slots[b]` and return float32 logits [n_wanted, vocab].
+
+        want: "last" (the last token of every sequence), "all", or for each sequence the places
+        among its new tokens.  Rows come in the order of the sequences and of `want`.
+        """
+        batch = self.prepare(slots, tokens, want)
+        if batch.n_tokens == 0:
+            return torch.empty(0, self.vocab, dtype=torch.float32, device=self.device)
+        return self.model.forward(batch, self.cache)
+
+    def prepare(self, slots, tokens, want) -> StepBatch:
+        slots = [int(s) for s in slots]
+        if len(slots) != len(tokens):
+            raise ValueError("one token list per sequence is needed")
+        if len(set(slots)) != len(slots):
+            raise ValueError("a sequence appears twice in one step")
+        for b, toks in enumerate(tokens):
+            if len(toks) == 0:
+                raise ValueError(f"sequence {b} of the step brings no token")
+            lo, hi = min(toks), max(toks)
+            if lo < 0 or hi >= self.vocab:
+                raise IndexError(f"token id {lo if lo < 0 else hi} is outside the vocabulary of {self.vocab}")
+        if want == "last":
+            want = [[len(t) - 1] for t in tokens]
+        elif want == "all":
+            want = [list(range(len(t))) for t in tokens]
+        elif len(want) != len(slots):
+            raise ValueError("one list of wanted places per sequence is needed")
+        # room for all, or for none
+        for group in self.cache.groups:
+            if group.need.window == 0:
+                need = sum(max(0, pages_for(self.cache.length(s) + len(t)) - len(group.pages[s])) for s, t in zip(slots, tokens))
+                if need > group.pool.n_free:
+                    raise CacheFull(f"the step needs {need} more cache pages, {group.pool.n_free} are free")
+        for s, t in zip(slots, tokens):
+            if self.cache.length(s) + len(t) > self.cache.max_seq_len:
+                raise IndexError(f"sequence in slot {s} would reach {self.cache.length(s) + len(t)} tokens; the model has {self.cache.max_seq_len} positions")
+        starts = [self.cache.extend(s, len(t)) for s, t in zip(slots, tokens)]
+        return build_batch(self.cache, slots, tokens, starts, want, self.device, self.qblock)

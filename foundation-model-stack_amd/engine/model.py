@@ -1,0 +1,86 @@
+"""A decoder model assembled from a ``ModelSpec``: embedding, layers run in the
+order of the schedule, final norm, head.  It knows no architecture by name."""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..cache import KVNeed, SequenceCache, StateNeed
+from ..parts import LayerCache, ModelSpec, Part, ResidualStream, make_part
+
+
+class DecoderModel(Part):
+    def __init__(self, spec: ModelSpec, dtype: torch.dtype, config=None):
+        super().__init__()
+        if dtype not in (torch.float32, torch.bfloat16):
+            raise TypeError(f"models run in float32 or bfloat16, not {dtype}")
+        self.spec, self.dtype, self.config = spec, dtype, config
+        self.device: Optional[torch.device] = None
+        self.schedule = spec.resolved_schedule()
+
+        self.positions = {name: make_part("position", p.kind, **p.args) for name, p in spec.positions.items()}
+        self.embedding = self.add_child(spec.embedding_name, make_part("embedding", spec.embedding.kind, vocab=spec.vocab, width=spec.width, **spec.embedding.args))
+        self.layers: List[Part] = []
+        for i, layer in enumerate(spec.layers):
+            pos = self.positions[layer.position] if layer.position is not None else None
+            mixer = make_part("mixer", layer.mixer.kind, width=spec.width, position_encoder=pos, **layer.mixer.args)
+            ff = make_part("feed_forward", layer.feed_forward.kind, width=spec.width, **layer.feed_forward.args)
+            norm1 = make_part("norm", layer.norm.kind, width=spec.width, **layer.norm.args)
+            norm2 = make_part("norm", layer.norm.kind, width=spec.width, **layer.norm.args)
+            block = make_part("block", layer.block.kind, mixer=mixer, feed_forward=ff, norm1=norm1, norm2=norm2, **layer.block.args)
+            self.layers.append(self.add_child(spec.layer_name.format(i=i), block))
+        self.final_norm = self.add_child(spec.final_norm_name, make_part("norm", spec.final_norm.kind, width=spec.width, **spec.final_norm.args))
+        self.head = self.add_child(spec.head_name, make_part("head", spec.head.kind, width=spec.width, vocab=spec.vocab, **spec.head.args))
+        # with tied heads the head's table is the embedding's (fms/models/llama.py:414-423)
+        self.tied = {}
+        if spec.tie_heads:
+            self.tied[spec.head_name + ".weight"] = spec.embedding_name + ".weight"
+
+    # ---- what the model asks of a cache ------------------------------------
+    def cache_needs(self) -> Tuple[List[Tuple[int, KVNeed]], List[Tuple[int, StateNeed]]]:
+        kv, state = [], []
+        for n, entry in enumerate(self.schedule):
+            mixer = self.layers[entry.layer].mixer
+            need = mixer.kv_need()
+            if need is not None and entry.cache_of is None:
+                kv.append((n, need))
+            if entry.cache_of is not None:
+                other = self.layers[self.schedule[entry.cache_of].layer].mixer.kv_need()
+                if need is None or other != need:
+                    raise ValueError(f"schedule entry {n} cannot read the cache of entry {entry.cache_of}: their needs differ")
+            sneed = mixer.state_need()
+            if sneed is not None:
+                state.append((n, sneed))
+        return kv, state
+
+    def make_cache(self, max_tokens: int, max_slots: int, device=None) -> SequenceCache:
+        kv, state = self.cache_needs()
+        return SequenceCache(kv, state, max_tokens, max_slots, self.spec.max_seq_len, self.dtype,
+                             self.device if device is None else device)
+
+    def finalize_all(self, device) -> None:
+        self.device = torch.device(device)
+        for part in self.walk():
+            part.finalize(self.device, self.dtype)
+        for part in self.positions.values():
+            part.finalize(self.device, self.dtype)
+
+    # ---- one pass over the tokens of a step --------------------------------
+    def forward(self, batch, cache: SequenceCache) -> torch.Tensor:
+        """float32 logits [n wanted rows, vocab] of the tokens in `batch`; the cache is extended in place."""
+        max_position = batch.max_context - 1
+        stream = ResidualStream(self.embedding.forward(batch.token_ids))
+        for n, entry in enumerate(self.schedule):
+            block = self.layers[entry.layer]
+            block.mixer.check_step(max_position)
+            owner = n if entry.cache_of is None else entry.cache_of
+            if owner in cache.group_of_entry:
+                group, keys, values = cache.kv_of_entry(owner)
+            else:
+                group, keys, values = -1, None, None
+            view = LayerCache(group, keys, values, entry.cache_of is None, cache.state_of_entry(n))
+            block.forward(stream, batch, view, self.dtype)
+        normed = self.final_norm.add_norm(stream.resid, stream.pending, self.dtype, rows=batch.logit_rows)
+        return self.head.forward(normed)

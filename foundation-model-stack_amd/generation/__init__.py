@@ -1,0 +1,11 @@
+from .loop import (
+    default_engine,
+    generate,
+    generate_requests,
+    pad_input_ids,
+    plan_batches,
+    trim_prefix,
+    truncate_after_eos,
+)
+
+__all__ = ["default_engine", "generate", "generate_requests", "pad_input_ids", "plan_batches", "trim_prefix", "truncate_after_eos"]

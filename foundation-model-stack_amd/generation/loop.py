@@ -1,0 +1,284 @@
+"""The generation loop above the step function.
+
+``generate_requests`` takes any number of prompts of unequal lengths, runs them
+in as many batches as the cache has room for, one batch after another; in a
+batch the prompts go through in one step, then every sequence still alive gets
+one token per step.  A sequence ends at a stop token, at max_new_tokens, or at
+the model's last position; its slot goes back at once and the batch shrinks.
+
+``generate`` has the reference's signature and meanings
+(fms/utils/generation.py:182-369) on top of that.
+"""
+
+from __future__ import annotations
+
+import time
+from typing import Callable, Iterable, List, Optional, Sequence, Set, Union
+
+import torch
+
+from ..cache import PAGE_TOKENS, pages_for
+from ..sampling import SamplingParams, choose, request_seed
+
+
+def plan_batches(
+    prompt_lens: Sequence[int],
+    max_new_tokens: int,
+    max_tokens: int,
+    max_batch: int,
+    max_seq_len: int,
+) -> List[List[int]]:
+    """Split requests (by index, in order) into batches that fit the cache.
+
+    A request may grow to min(prompt + max_new_tokens, max_seq_len) tokens, rounded up to a
+    page; a batch holds as many consecutive requests as fit into max_tokens and max_batch.
+    """
+    batches: List[List[int]] = []
+    current: List[int] = []
+    used = 0
+    for i, n in enumerate(prompt_lens):
+        if n <= 0:
+            raise ValueError(f"request {i} has an empty prompt")
+        if n > max_seq_len:
+            raise IndexError(f"request {i} has {n} prompt tokens, the model has {max_seq_len} positions")
+        need = pages_for(min(n + max_new_tokens, max_seq_len)) * PAGE_TOKENS
+        if need > max_tokens:
+            raise ValueError(f"request {i} may need {need} cached tokens, the cache holds {max_tokens}")
+        if current and (used + need > max_tokens or len(current) >= max_batch):
+            batches.append(current)
+            current, used = [], 0
+        current.append(i)
+        used += need
+    if current:
+        batches.append(current)
+    return batches
+
+
+def generate_requests(
+    engine,
+    prompts: Sequence[Sequence[int]],
+    max_new_tokens: int = 256,
+    sampling: Optional[SamplingParams] = None,
+    stop_token_ids: Optional[Iterable[int]] = None,
+    seed: int = 0,
+    max_batch: Optional[int] = None,
+    chooser: Optional[Callable] = None,
+    on_step: Optional[Callable[[int, List[int], List[int]], None]] = None,
+    step_times: Optional[List[float]] = None,
+) -> List[List[int]]:
+    """New tokens of every request (a stop token is kept, nothing follows it).
+
+    engine: anything with new_sequence(), end_sequence(slot), step(slots, tokens, want), and
+    cache.max_tokens / cache.max_slots / cache.max_seq_len.  chooser(logits, request_indices,
+    counters) -> token ids overrides the built-in sampler (tests use it).
+    """
+    sampling = sampling or SamplingParams(do_sample=False)
+    stops: Set[int] = set(int(s) for s in (stop_token_ids or ()))
+    prompts = [list(map(int, p)) for p in prompts]
+    results: List[List[int]] = [[] for _ in prompts]
+    if max_new_tokens <= 0 or not prompts:
+        return results
+    cache = engine.cache
+    max_batch = min(max_batch or cache.max_slots, cache.max_slots)
+
+    def pick(logits, request_ids, counters) -> List[int]:
+        if chooser is not None:
+            return [int(t) for t in chooser(logits, request_ids, counters)]
+        seeds = [request_seed(seed, r) for r in request_ids]
+        return choose(logits, sampling, seeds, counters).tolist()
+
+    for batch in plan_batches([len(p) for p in prompts], max_new_tokens, cache.max_tokens, max_batch, cache.max_seq_len):
+        slots = {r: engine.new_sequence() for r in batch}
+        alive = list(batch)
+        feed = {r: prompts[r] for r in batch}
+        step_no = 0
+        try:
+            while alive:
+                t0 = time.time()
+                logits = engine.step([slots[r] for r in alive], [feed[r] for r in alive], "last")
+                tokens = pick(logits, alive, [len(results[r]) for r in alive])
+                if step_times is not None:
+                    step_times.append(time.time() - t0)
+                if on_step is not None:
+                    on_step(step_no, list(alive), list(tokens))
+                still = []
+                for r, tok in zip(alive, tokens):
+                    results[r].append(tok)
+                    length = len(prompts[r]) + len(results[r])
+                    # the token just chosen is not in the cache yet: it may be fed only if a position is left for it
+                    done = tok in stops or len(results[r]) >= max_new_tokens or length > cache.max_seq_len
+                    if done:
+                        engine.end_sequence(slots.pop(r))
+                    else:
+                        feed[r] = [tok]
+                        still.append(r)
+                alive = still
+                step_no += 1
+        finally:
+            for slot in slots.values():
+                engine.end_sequence(slot)
+    return results
+
+
+# --------------------------------------------------------------------------
+# the reference's call
+# --------------------------------------------------------------------------
+def pad_input_ids(input_ids_list: List[torch.Tensor], min_pad_length: int = 0, is_causal_mask=True,
+                  padding_side="left", position_ids_offset=0, pad_token_id=0):
+    """A rectangular tensor from prompts of unequal lengths, with the mask and position_ids the
+    reference builds (fms/utils/generation.py:16-109).  ``generate`` reads the real lengths back
+    from ``position_ids``/``mask``; the engine itself never sees padding."""
+    max_len = max([min_pad_length] + [seq.size(0) for seq in input_ids_list])
+    rows, masks, positions = [], [], []
+    for seq in input_ids_list:
+        n = seq.size(0)
+        pads = torch.full((max_len - n,), pad_token_id, dtype=torch.long, device=seq.device)
+        real = torch.ones(n, dtype=torch.bool, device=seq.device)
+        fake = torch.zeros(max_len - n, dtype=torch.bool, device=seq.device)
+        pos_pad = torch.zeros(max_len - n, dtype=torch.long, device=seq.device)
+        pos = torch.arange(0, n, dtype=torch.long, device=seq.device)
+        if padding_side == "left":
+            rows.append(torch.cat((pads, seq)))
+            masks.append(torch.cat((fake, real)))
+            positions.append(torch.cat((pos_pad, pos)))
+        elif padding_side == "right":
+            rows.append(torch.cat((seq, pads)))
+            masks.append(torch.cat((real, fake)))
+            positions.append(torch.cat((pos, pos_pad)))
+        else:
+            raise NotImplementedError("padding_side must be 'right' or left'")
+    input_ids = torch.stack(rows)
+    mask = torch.stack(masks)
+    mask = mask.unsqueeze(-1) == mask.unsqueeze(-2)
+    if is_causal_mask:
+        mask = mask.tril()
+    mask = torch.where(mask.logical_not(), -torch.inf, 0.0)
+    position_ids = torch.stack(positions) + position_ids_offset
+    return input_ids, {
+        "mask": mask,
+        "position_ids": position_ids,
+        "lengths": [seq.size(0) for seq in input_ids_list],
+        "padding_side": padding_side,
+    }
+
+
+def _real_tokens(input_ids: torch.Tensor, extra_kwargs) -> List[List[int]]:
+    """Rows of a rectangular batch without their padding.
+
+    pad_input_ids records the real lengths and the padding side; a mask from elsewhere is read
+    as left padding, where the last row of a sequence's mask is open exactly at its real tokens.
+    """
+    rows = input_ids.tolist()
+    extra = extra_kwargs or {}
+    if "lengths" in extra:
+        side = extra.get("padding_side", "left")
+        return [row[len(row) - n :] if side == "left" else row[:n] for row, n in zip(rows, extra["lengths"])]
+    mask = extra.get("mask")
+    if mask is None:
+        return rows
+    return [[tok for tok, keep in zip(row, (mask[b][-1] == 0).tolist()) if keep] for b, row in enumerate(rows)]
+
+
+def generate(
+    model,
+    input_ids: torch.Tensor,
+    max_seq_len: int = 4096,
+    max_new_tokens: int = 256,
+    temperature: float = 1.0,
+    top_k: int = 10,
+    do_sample: bool = True,
+    num_beams: int = 1,
+    use_cache: bool = True,
+    contiguous_cache: bool = False,
+    eos_token_id: Optional[int] = None,
+    pad_token_id: Optional[int] = None,
+    timing: str = "",
+    post_iteration_hook: Optional[Callable] = None,
+    extra_kwargs: Optional[dict] = None,
+    seed: int = 0,
+):
+    """The reference's generate (fms/utils/generation.py:182-369) on this engine.
+
+    input_ids: a 1-D tensor (one prompt) or a 2-D tensor (a batch; rows padded by pad_input_ids
+    carry their mask in extra_kwargs).  Returns prompt + generated tokens, [S + n] or [B, S + n];
+    a row that ended early is filled up with eos_token_id (or pad_token_id, or 0).
+    use_cache / contiguous_cache are accepted for compatibility: the engine always caches.
+    With timing "per-token" or "e2e" returns (result, times) as the reference does.
+    """
+    from ..engine import Engine  # late import: engine imports the kernels
+
+    if num_beams != 1:
+        raise NotImplementedError("generate() does yet not support beam search")
+    if not isinstance(input_ids, torch.Tensor):
+        raise TypeError("input_ids must be one of Tensor or List")
+    is_batch = input_ids.dim() > 1
+    ids2d = input_ids if is_batch else input_ids.unsqueeze(0)
+    prompts = _real_tokens(ids2d.cpu(), extra_kwargs)
+    prompts = [p[-max_seq_len:] for p in prompts]
+
+    engine = model if isinstance(model, Engine) else default_engine(model, prompts, max_new_tokens)
+    times: List[float] = []
+    start = time.time()
+    hook = None
+    if post_iteration_hook is not None:
+        hook = lambda step, alive, tokens: post_iteration_hook(step, alive, tokens)  # noqa: E731
+    new = generate_requests(
+        engine,
+        prompts,
+        max_new_tokens=max_new_tokens,
+        sampling=SamplingParams(do_sample=do_sample, temperature=temperature, top_k=top_k or 0),
+        stop_token_ids=None if eos_token_id is None else [eos_token_id],
+        seed=seed,
+        on_step=hook,
+        step_times=times if timing == "per-token" else None,
+    )
+    if timing == "e2e":
+        if engine.device.type == "cuda":
+            torch.cuda.synchronize()
+        times = [time.time() - start]
+    fill = eos_token_id if eos_token_id is not None else (pad_token_id if pad_token_id is not None else 0)
+    width = max(len(n) for n in new) if new else 0
+    rows = []
+    for b in range(ids2d.shape[0]):
+        tail = new[b] + [fill] * (width - len(new[b]))
+        rows.append(torch.cat((ids2d[b].cpu(), torch.tensor(tail, dtype=ids2d.dtype))))
+    result = torch.stack(rows).to(input_ids.device)
+    if not is_batch:
+        result = result[0]
+    if timing != "":
+        return result, times
+    return result
+
+
+def default_engine(model, prompts, max_new_tokens):
+    """An engine for `model` with room for these requests, kept on the model and reused while it is large enough."""
+    from ..engine import Engine
+
+    need = sum(pages_for(min(len(p) + max_new_tokens, model.spec.max_seq_len)) for p in prompts) * PAGE_TOKENS
+    engine = getattr(model, "_default_engine", None)
+    if engine is None or engine.cache.max_tokens < need or engine.cache.max_slots < len(prompts):
+        engine = Engine(model, max_tokens=need, max_slots=max(len(prompts), 1))
+        model._default_engine = engine
+    return engine
+
+
+def truncate_after_eos(result: torch.Tensor, eos_token_id) -> torch.Tensor:
+    """Cut a 1-D result after its first eos token (fms/utils/generation.py:372-387)."""
+    if eos_token_id is None:
+        return result
+    idx = torch.where(result == eos_token_id)[0]
+    if idx.shape[0] >= 1:
+        result = result[: idx[0] + 1]
+    return result
+
+
+def trim_prefix(result: torch.Tensor, pad_token_id: int = 0) -> torch.Tensor:
+    """Drop leading pad tokens and the token that follows them... as the reference does
+    (fms/utils/generation.py:390-413): everything up to and including the last leading pad."""
+    if result[0] != pad_token_id:
+        return result
+    diff = (result != pad_token_id).diff()
+    first = torch.where(diff > 0)[0]
+    if first.numel() == 0:
+        return result
+    return result[first[0] + 1 :]

@@ -1,0 +1,88 @@
+"""Multi-head attention with grouped kv heads over the paged cache: the mixer of Llama.
+
+The reference's order of operations (fms/modules/attention.py:870-937): one fused
+projection split into [H*D | K*D | K*D]; rotate queries and keys; append keys and
+values to the cache; causal scaled-dot-product attention in which query head h reads
+kv head h // (H/K) (:241-250) with scale 1/sqrt(D) unless given (:768-784); output
+projection.  Here the rotation and the cache append are one kernel, and attention
+reads the cache directly, so a step may bring any number of new tokens per sequence.
+"""
+
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from ..cache import KVNeed
+from ..kernels import ops
+from .base import Mixer, Part, register_part
+from .linear import Linear
+from .position import PositionEncoding
+
+
+class LayerCache:
+    """What a mixer sees of the cache for one schedule entry."""
+
+    def __init__(self, group: int, keys: Optional[torch.Tensor], values: Optional[torch.Tensor], owns: bool, state: dict):
+        self.group, self.keys, self.values, self.owns, self.state = group, keys, values, owns, state
+
+
+class MultiHeadAttention(Mixer):
+    def __init__(
+        self,
+        width: int,
+        nheads: int,
+        kvheads: int,
+        head_dim: int,
+        use_bias: bool = False,
+        position_encoder: Optional[PositionEncoding] = None,
+        scale_factor: Optional[float] = None,
+        window: int = 0,
+    ):
+        super().__init__()
+        if kvheads <= 0 or nheads % kvheads:
+            raise ValueError(f"{nheads} query heads are no multiple of {kvheads} kv heads")
+        if head_dim % 2 or head_dim > 256:
+            raise ValueError(f"head size {head_dim} must be even and at most 256")
+        self.width, self.nheads, self.kvheads, self.head_dim = width, nheads, kvheads, head_dim
+        self.scale = float(scale_factor) if scale_factor is not None else 1.0 / math.sqrt(head_dim)
+        self.window = int(window)
+        self.position_encoder = position_encoder
+        in_proj = self.add_child("in_proj", Part())
+        self.qkv = in_proj.add_child("qkv_fused", Linear(width, (nheads + 2 * kvheads) * head_dim, use_bias))
+        self.dense = self.add_child("dense", Linear(nheads * head_dim, width, use_bias))
+
+    # ---- what the mixer asks of the cache ---------------------------------
+    def kv_need(self) -> Optional[KVNeed]:
+        return KVNeed(self.kvheads, self.head_dim, self.window)
+
+    def state_need(self):
+        return None
+
+    def check_step(self, max_position: int) -> None:
+        if self.position_encoder is not None:
+            self.position_encoder.check_positions(max_position)
+
+    def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
+        H, K, D = self.nheads, self.kvheads, self.head_dim
+        qkv = self.qkv.forward(x)
+        table = batch.block_tables[cache.group]
+        tables = self.position_encoder.rotary_tables() if self.position_encoder is not None else None
+        if tables is None and self.position_encoder is not None:
+            self.position_encoder.adjust_qk(qkv, batch, H, K, D)
+        cos, sin, rot = tables if tables is not None else (None, None, 0)
+        ops.rope_kv_write(
+            qkv, batch.positions, batch.seq_of_token, table, cos, sin, rot,
+            cache.keys if cache.owns else None, cache.values if cache.owns else None, H, K, D,
+        )
+        mixed = ops.attention(
+            qkv, batch.positions, batch.seq_of_token, table, cache.keys, cache.values, H, K, D, self.scale, self.window,
+            decode=batch.is_decode, max_context=batch.max_context,
+            qblock_start=batch.qblock_start, qblock_len=batch.qblock_len,
+        )
+        return self.dense.forward(mixed)
+
+
+register_part("mixer", "attention", MultiHeadAttention)

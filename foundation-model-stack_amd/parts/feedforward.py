@@ -1,0 +1,31 @@
+"""Feed-forward parts.
+
+``GatedLinearUnit`` is the reference's SwiGLU (fms/modules/feedforward.py:193-327):
+one fused projection whose first half is the gate and second half the "up" path
+(:288-297), out = w2(act(gate) * up).
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import FeedForward, register_part
+from .linear import Linear
+
+
+class GatedLinearUnit(FeedForward):
+    def __init__(self, width: int, hidden_dim: int, activation: str = "swish", use_bias: bool = False):
+        super().__init__()
+        if activation not in ops.ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not one of {sorted(ops.ACTIVATIONS)}")
+        self.width, self.hidden_dim, self.activation = width, int(hidden_dim), activation
+        self.wg1 = self.add_child("wg1_fused", Linear(width, 2 * self.hidden_dim, use_bias))
+        self.w2 = self.add_child("w2", Linear(self.hidden_dim, width, use_bias))
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        hidden = ops.gated_linear(x, self.wg1.w["weight"], self.wg1.w.get("bias"), self.activation)
+        return self.w2.forward(hidden)
+
+
+register_part("feed_forward", "glu", GatedLinearUnit)

@@ -1,0 +1,48 @@
+"""The parameterised norm of the reference (fms/modules/layernorm.py:5-69).
+
+Llama uses it as RMSNorm: no mean subtraction, a learned scale, no shift, eps
+inside the root.  Statistics, scaling and the multiplication by the weight are
+float32; the result is rounded once to the activation type.  The kernel also
+folds in the residual addition that precedes the norm in a pre-norm block.
+"""
+
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..kernels import ops
+from .base import Part, register_part
+
+
+class ParameterizedNorm(Part):
+    def __init__(
+        self,
+        width: int,
+        eps: float = 1e-6,
+        elementwise_scale: bool = True,
+        elementwise_shift: bool = False,
+        use_mean: bool = False,
+    ):
+        super().__init__()
+        self.width, self.eps, self.use_mean = width, float(eps), use_mean
+        if elementwise_scale:
+            self.declare("weight", (width,), init="ones")
+        if elementwise_shift:
+            self.declare("bias", (width,), init="zeros")
+
+    def add_norm(
+        self,
+        resid: torch.Tensor,
+        branch: Optional[torch.Tensor],
+        out_dtype: torch.dtype,
+        rows: Optional[torch.Tensor] = None,
+    ) -> torch.Tensor:
+        """resid += branch (float32, in place); returns norm(resid) in out_dtype (only `rows` if given)."""
+        return ops.add_norm(resid, branch, self.w.get("weight"), self.w.get("bias"), self.eps, out_dtype, rows, self.use_mean)
+
+
+register_part("norm", "rmsnorm", lambda width, eps=1e-6, **kw: ParameterizedNorm(width, eps, True, False, False, **kw))
+register_part("norm", "layernorm", lambda width, eps=1e-6, **kw: ParameterizedNorm(width, eps, True, True, True, **kw))
+register_part("norm", "parameterized", ParameterizedNorm)

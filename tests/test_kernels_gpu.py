@@ -1,0 +1,379 @@
+"""Each kernel alone against a plain float32 torch formula, at sizes other than the engine's."""
+
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import plain_llama as P  # noqa: E402
+
+PAGE = 64
+
+
+@pytest.fixture(scope="module")
+def ops():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from fms_amd.kernels import load, ops as _ops
+
+    load()
+    return _ops
+
+
+def dev(t):
+    return t.to("cuda")
+
+
+def tol(dtype):
+    return dict(atol=2e-5, rtol=2e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+
+
+# --------------------------------------------------------------------------
+def test_embed(ops):
+    torch.manual_seed(0)
+    for dtype in (torch.float32, torch.bfloat16):
+        table = torch.randn(37, 24).to(dtype)
+        ids = torch.tensor([0, 36, 5, 5, 17], dtype=torch.int32)
+        out = ops.embed(dev(ids), dev(table)).cpu()
+        assert out.dtype == torch.float32
+        assert torch.equal(out, table.float()[ids.long()])
+
+
+@pytest.mark.parametrize("width", [24, 100, 4096, 9000])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_add_norm(ops, width, dtype):
+    torch.manual_seed(1)
+    T = 5
+    resid = torch.randn(T, width) * 2
+    branch = torch.randn(T, width).to(dtype)
+    weight = (1 + 0.3 * torch.randn(width)).to(dtype)
+    eps = 1e-3
+    want_resid = resid + branch.float()
+    want = P.rms_norm(want_resid, weight.float(), eps)
+    r = dev(resid.clone())
+    out = ops.add_norm(r, dev(branch), dev(weight), None, eps, dtype)
+    torch.testing.assert_close(r.cpu(), want_resid)
+    torch.testing.assert_close(out.cpu().float(), want, **tol(dtype))
+    # no branch; selected rows only; the stream is left alone
+    r2 = dev(resid.clone())
+    rows = torch.tensor([3, 0], dtype=torch.int32)
+    out2 = ops.add_norm(r2, dev(branch), dev(weight), None, eps, dtype, rows=dev(rows))
+    torch.testing.assert_close(out2.cpu().float(), want[rows.long()], **tol(dtype))
+    assert torch.equal(r2.cpu(), resid)
+    out3 = ops.add_norm(dev(resid.clone()), None, dev(weight), None, eps, dtype)
+    torch.testing.assert_close(out3.cpu().float(), P.rms_norm(resid, weight.float(), eps), **tol(dtype))
+
+
+def test_add_norm_with_mean_and_shift(ops):
+    torch.manual_seed(2)
+    x = torch.randn(3, 48) + 1.5
+    w, b = torch.randn(48), torch.randn(48)
+    out = ops.add_norm(dev(x.clone()), None, dev(w), dev(b), 1e-5, torch.float32, use_mean=True)
+    torch.testing.assert_close(out.cpu(), torch.nn.functional.layer_norm(x, (48,), w, b, 1e-5), atol=1e-5, rtol=1e-5)
+    # a float32 weight with bfloat16 activations (a tensor the checkpoint keeps in 32-bit)
+    out = ops.add_norm(dev(x.clone()), None, dev(w), None, 1e-5, torch.bfloat16)
+    torch.testing.assert_close(out.cpu().float(), P.rms_norm(x, w, 1e-5), atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gated_act(ops, dtype):
+    torch.manual_seed(3)
+    gu = torch.randn(7, 2 * 44).to(dtype)
+    bias = torch.randn(2 * 44).to(dtype)
+    out = ops.gated_act(dev(gu), dev(bias), "swish").cpu().float()
+    g = gu.float() + bias.float()
+    torch.testing.assert_close(out, P.silu(g[:, :44]) * g[:, 44:], **tol(dtype))
+    out = ops.gated_act(dev(gu), None, "silu").cpu().float()
+    torch.testing.assert_close(out, P.silu(gu.float()[:, :44]) * gu.float()[:, 44:], **tol(dtype))
+
+
+def test_cast_and_bias(ops):
+    x = torch.randn(1000)
+    assert torch.equal(ops.cast(dev(x), torch.bfloat16).cpu(), x.to(torch.bfloat16))
+    assert torch.equal(ops.cast(dev(x.to(torch.bfloat16)), torch.float32).cpu(), x.to(torch.bfloat16).float())
+    m = torch.randn(4, 10)
+    b = torch.randn(10)
+    torch.testing.assert_close(ops.bias_add_(dev(m.clone()), dev(b)).cpu(), m + b)
+
+
+def test_rope_table(ops):
+    freqs = P.rope_frequencies(24, 500000.0)
+    cos, sin = ops.rope_table(dev(freqs), 300)
+    angles = torch.outer(torch.arange(300).float(), freqs)
+    torch.testing.assert_close(cos.cpu(), torch.cos(angles), atol=2e-6, rtol=0)
+    torch.testing.assert_close(sin.cpu(), torch.sin(angles), atol=2e-6, rtol=0)
+    # large angles keep their accuracy (positions in the thousands times frequency one)
+    cos, sin = ops.rope_table(dev(torch.tensor([1.0, 0.37])), 9000)
+    a = torch.outer(torch.arange(9000).float(), torch.tensor([1.0, 0.37]))
+    torch.testing.assert_close(cos.cpu(), torch.cos(a.double()).float(), atol=5e-7, rtol=0)
+
+
+# --------------------------------------------------------------------------
+# paged cache helpers
+# --------------------------------------------------------------------------
+def make_pages(lengths, K, D, dtype, seed=0, extra_pages=3):
+    """Random page assignment: returns (block_table [B, P] int32, n_pages)."""
+    g = torch.Generator().manual_seed(seed)
+    per_seq = [-(-n // PAGE) for n in lengths]
+    total = sum(per_seq) + extra_pages
+    perm = torch.randperm(total, generator=g).tolist()
+    width = max(per_seq)
+    table = torch.full((len(lengths), width), -1, dtype=torch.int32)
+    it = iter(perm)
+    for b, n in enumerate(per_seq):
+        for i in range(n):
+            table[b, i] = next(it)
+    return table, total
+
+
+def fill_cache(table, ks, vs, n_pages, dtype):
+    """ks[b]: [len, K, D] -> caches in the kernels' layout."""
+    K, D = ks[0].shape[1:]
+    kc = torch.zeros(n_pages, K, PAGE, D, dtype=dtype)
+    vc = torch.zeros(n_pages, K, D, PAGE, dtype=dtype)
+    for b, (k, v) in enumerate(zip(ks, vs)):
+        for pos in range(k.shape[0]):
+            page = int(table[b, pos // PAGE])
+            kc[page, :, pos % PAGE, :] = k[pos].to(dtype)
+            vc[page, :, :, pos % PAGE] = v[pos].to(dtype)
+    return kc, vc
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,K,D,rot", [(4, 2, 16, 16), (3, 1, 24, 24), (2, 2, 32, 16)])
+def test_rope_kv_write(ops, dtype, H, K, D, rot):
+    torch.manual_seed(4)
+    starts, lens = [0, 70, 5], [9, 3, 130]
+    total = [s + n for s, n in zip(starts, lens)]
+    table, n_pages = make_pages(total, K, D, dtype, seed=1)
+    T = sum(lens)
+    qkv = torch.randn(T, (H + 2 * K) * D).to(dtype)
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int()
+    seq = torch.cat([torch.full((n,), b) for b, n in enumerate(lens)]).int()
+    freqs = P.rope_frequencies(rot, 10000.0)
+    cos, sin = ops.rope_table(dev(freqs), 256)
+    kc = torch.zeros(n_pages, K, PAGE, D, dtype=dtype, device="cuda")
+    vc = torch.zeros(n_pages, K, D, PAGE, dtype=dtype, device="cuda")
+    q_dev = dev(qkv.clone())
+    ops.rope_kv_write(q_dev, dev(positions), dev(seq), dev(table), cos, sin, rot, kc, vc, H, K, D)
+    out = q_dev.cpu().float()
+    x = qkv.float()
+    q = x[:, : H * D].reshape(T, H, D)
+    k = x[:, H * D : (H + K) * D].reshape(T, K, D)
+    v = x[:, (H + K) * D :].reshape(T, K, D)
+
+    def rotate(t):
+        r = P.rope_rotate(t[..., :rot], positions, freqs)
+        return torch.cat([r, t[..., rot:]], dim=-1)
+
+    torch.testing.assert_close(out[:, : H * D].reshape(T, H, D), rotate(q), **tol(dtype))
+    # v columns of qkv untouched
+    assert torch.equal(out[:, (H + K) * D :], x[:, (H + K) * D :])
+    kc, vc = kc.cpu().float(), vc.cpu().float()
+    rk = rotate(k)
+    for t in range(T):
+        page = int(table[int(seq[t]), int(positions[t]) // PAGE])
+        off = int(positions[t]) % PAGE
+        torch.testing.assert_close(kc[page, :, off, :], rk[t], **tol(dtype))
+        torch.testing.assert_close(vc[page, :, :, off], v[t].to(dtype).float(), **tol(dtype))
+    # pages of no sequence stay zero: nothing was written elsewhere
+    used = set(int(p) for p in table.flatten() if p >= 0)
+    for p in range(n_pages):
+        if p not in used:
+            assert float(kc[p].abs().sum()) == 0 and float(vc[p].abs().sum()) == 0
+
+
+# --------------------------------------------------------------------------
+def reference_attention(qs, ks, vs, starts, H, K, scale=None, window=0):
+    """qs[b]: [n_b, H, D] queries at positions starts[b]..; ks/vs[b]: [len_b, K, D] all keys."""
+    outs = []
+    for q, k, v, s in zip(qs, ks, vs, starts):
+        n = q.shape[0]
+        full_q = torch.zeros(k.shape[0], H, q.shape[2])
+        full_q[s : s + n] = q
+        o = P.causal_attention(full_q, k.float(), v.float(), scale=scale, window=window)
+        outs.append(o[s : s + n])
+    return torch.cat(outs).reshape(sum(q.shape[0] for q in qs), -1)
+
+
+def attention_case(ops, dtype, H, K, D, starts, lens, window=0, decode=False, scale=None, spike=False, **kw):
+    torch.manual_seed(5)
+    totals = [s + n for s, n in zip(starts, lens)]
+    table, n_pages = make_pages(totals, K, D, dtype, seed=2)
+    ks = [torch.randn(n, K, D).to(dtype).float() for n in totals]
+    vs = [torch.randn(n, K, D).to(dtype).float() for n in totals]
+    qs = [torch.randn(n, H, D).to(dtype).float() for n in lens]
+    if spike:
+        # one far key decides the result: a kernel that loses it (a split, a page, a mask edge) fails visibly
+        for b in range(len(lens)):
+            far = totals[b] // 3
+            qs[b][-1, :, :] = 0
+            qs[b][-1, :, 0] = 8.0
+            ks[b][:, :, 0] = -1.0
+            ks[b][far, :, 0] = 8.0
+    kc, vc = fill_cache(table, ks, vs, n_pages, dtype)
+    T = sum(lens)
+    q_flat = torch.cat([q.reshape(q.shape[0], H * D) for q in qs]).to(dtype)
+    # queries sit inside wider rows, as in the fused qkv buffer
+    wide = torch.zeros(T, (H + 2 * K) * D, dtype=dtype)
+    wide[:, : H * D] = q_flat
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int()
+    seq = torch.cat([torch.full((n,), b) for b, n in enumerate(lens)]).int()
+    qblock = ops.prefill_qblock()
+    qb_start, qb_len, base = [], [], 0
+    for n in lens:
+        for off in range(0, n, qblock):
+            qb_start.append(base + off)
+            qb_len.append(min(qblock, n - off))
+        base += n
+    sc = scale if scale is not None else 1 / math.sqrt(D)
+    out = ops.attention(
+        dev(wide), dev(positions), dev(seq), dev(table), dev(kc), dev(vc), H, K, D, sc, window,
+        decode=decode, max_context=max(totals),
+        qblock_start=dev(torch.tensor(qb_start, dtype=torch.int32)), qblock_len=dev(torch.tensor(qb_len, dtype=torch.int32)), **kw,
+    )
+    want = reference_attention(qs, ks, vs, starts, H, K, scale=sc, window=window)
+    torch.testing.assert_close(out.cpu().float(), want, **(dict(atol=3e-5, rtol=3e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)))
+
+
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 24), (3, 3, 40), (2, 1, 8)])
+def test_attention_generic_f32(ops, H, K, D):
+    attention_case(ops, torch.float32, H, K, D, starts=[0, 0, 60], lens=[70, 1, 9])
+    attention_case(ops, torch.float32, H, K, D, starts=[299, 64], lens=[1, 1], decode=True)
+
+
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (6, 3, 128), (2, 2, 64), (32, 1, 32), (2, 1, 256), (5, 5, 80)])
+def test_attention_prefill_bf16(ops, H, K, D):
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 0, 0], lens=[200, 1, 33])
+    # a chunk that continues a cached prefix
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[100, 64, 0], lens=[70, 5, 129])
+
+
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (8, 2, 128), (2, 2, 64), (40, 2, 32), (2, 1, 256), (5, 5, 80)])
+def test_attention_decode_bf16(ops, H, K, D):
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 63, 64, 700], lens=[1, 1, 1, 1], decode=True)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=2)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=5)
+
+
+@pytest.mark.parametrize("dtype,decode", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
+def test_attention_far_key_and_window(ops, dtype, decode):
+    lens = [1, 1] if decode else [40, 3]
+    attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, spike=True)
+    attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=100)
+    attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=64, scale=0.3)
+    attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=1)
+
+
+def test_attention_generic_bf16_agrees(ops):
+    attention_case(ops, torch.bfloat16, 4, 2, 16, starts=[0, 10], lens=[70, 3], force_generic=True)
+
+
+# --------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K", [(1, 40, 24), (5, 100, 176), (64, 64, 64), (130, 257, 96), (70, 4096, 40)])
+def test_gemm_f32(ops, M, N, K):
+    torch.manual_seed(6)
+    x, w, b = torch.randn(M, K), torch.randn(N, K), torch.randn(N)
+    out = ops.linear(dev(x), dev(w), dev(b)).cpu()
+    torch.testing.assert_close(out, (x.double() @ w.double().t() + b.double()).float(), atol=1e-4, rtol=1e-5)
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 48, 64, 65, 200, 300])
+@pytest.mark.parametrize("N,K", [(40, 24), (100, 176), (384, 96), (4096 + 16, 512), (20000, 64)])
+def test_gemm_bf16(ops, M, N, K):
+    torch.manual_seed(7)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = (torch.randn(N, K) * 0.1).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16)
+    want = x.double() @ w.double().t()
+    for out_dtype in (torch.bfloat16, torch.float32):
+        for allow_library in (True, False):
+            out = ops.linear(dev(x), dev(w), None, out_dtype=out_dtype, allow_library=allow_library).cpu()
+            assert out.dtype == out_dtype
+            torch.testing.assert_close(out.double(), want, atol=3e-2 if out_dtype == torch.bfloat16 else 2e-3, rtol=1e-2)
+    out = ops.linear(dev(x), dev(w), dev(b), out_dtype=torch.float32, allow_library=False).cpu()
+    torch.testing.assert_close(out.double(), want + b.double(), atol=2e-3, rtol=1e-2)
+    # a float32 bias with bfloat16 weights, and a float32 weight with bfloat16 activations
+    out = ops.linear(dev(x), dev(w), dev(b.float()), out_dtype=torch.float32).cpu()
+    torch.testing.assert_close(out.double(), want + b.double(), atol=2e-3, rtol=1e-2)
+    out = ops.linear(dev(x), dev(w.float()), None).cpu()
+    assert out.dtype == torch.bfloat16
+    torch.testing.assert_close(out.double(), want, atol=3e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100])
+@pytest.mark.parametrize("hidden,K", [(44, 24), (176, 64), (1000, 96)])
+def test_gated_linear(ops, M, hidden, K):
+    torch.manual_seed(8)
+    for dtype in (torch.bfloat16, torch.float32):
+        x = torch.randn(M, K).to(dtype)
+        w = (torch.randn(2 * hidden, K) * 0.2).to(dtype)
+        b = torch.randn(2 * hidden).to(dtype)
+        for bias in (None, b):
+            out = ops.gated_linear(dev(x), dev(w), None if bias is None else dev(bias), "swish").cpu().float()
+            gu = x.float() @ w.float().t() + (0 if bias is None else bias.float())
+            want = P.silu(gu[:, :hidden]) * gu[:, hidden:]
+            torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=4e-2, rtol=2e-2)))
+
+
+# --------------------------------------------------------------------------
+def test_argmax(ops):
+    torch.manual_seed(9)
+    logits = torch.randn(6, 1000)
+    logits[2, 17] = logits[2, 900] = 50.0  # equal maxima: the lowest index wins
+    out = ops.sample(dev(logits), False).cpu()
+    want = logits.argmax(-1)
+    want[2] = 17
+    assert out.tolist() == want.tolist()
+    big = torch.randn(2, 128256)
+    assert ops.sample(dev(big), False).cpu().tolist() == big.argmax(-1).tolist()
+
+
+@pytest.mark.parametrize("vocab,top_k,temperature", [(50, 0, 1.0), (384, 10, 0.8), (5000, 3, 2.0), (128256, 50, 0.7), (300, 1000, 1.0)])
+def test_sampling(ops, vocab, top_k, temperature):
+    from fms_amd.sampling import uniform
+
+    torch.manual_seed(10)
+    rows = 64
+    logits = torch.randn(rows, vocab) * 3
+    seeds = [1234 + 7 * r for r in range(rows)]
+    counters = [r % 5 for r in range(rows)]
+    rng = torch.tensor([[s, c] for s, c in zip(seeds, counters)], dtype=torch.int64)
+    rng_dev = dev(rng)
+    out = ops.sample(dev(logits), True, temperature, top_k, rng_dev).cpu().tolist()
+    assert rng_dev.cpu()[:, 1].tolist() == [c + 1 for c in counters]
+    for r in range(rows):
+        p = P.sampling_distribution(logits[r], temperature, top_k).double()
+        cdf = torch.cumsum(p, 0)
+        u = uniform(seeds[r], counters[r])
+        tok = out[r]
+        assert p[tok] > 0, "a token outside the kept set was drawn"
+        lo = float(cdf[tok] - p[tok])
+        hi = float(cdf[tok])
+        assert lo - 1e-5 <= u <= hi + 1e-5, (r, tok, u, lo, hi)
+    if top_k == 3:
+        kept = [set(torch.topk(logits[r], 3).indices.tolist()) for r in range(rows)]
+        assert all(out[r] in kept[r] for r in range(rows))
+
+
+def test_sampling_ties_at_threshold_survive(ops):
+    logits = torch.full((1, 100), -5.0)
+    logits[0, [3, 50, 77]] = 2.0  # top_k=2 but three equal maxima: all three stay
+    seen = set()
+    for c in range(200):
+        rng = dev(torch.tensor([[99, c]], dtype=torch.int64))
+        seen.add(int(ops.sample(dev(logits), True, 1.0, 2, rng).cpu()[0]))
+    assert seen == {3, 50, 77}
+
+
+def test_kernels_refuse_what_they_cannot_do(ops):
+    from fms_amd.kernels import KernelError
+
+    with pytest.raises((KernelError, ValueError)):
+        ops.linear(dev(torch.zeros(2, 12, dtype=torch.bfloat16)), dev(torch.zeros(8, 12, dtype=torch.bfloat16)))  # K % 8
+    with pytest.raises(RuntimeError):
+        ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4))  # CPU tensors: no CPU path
+    with pytest.raises((KernelError, ValueError)):
+        ops.sample(dev(torch.zeros(1, 8)), True, 0.0, 0, dev(torch.zeros(1, 2, dtype=torch.int64)))

@@ -1,0 +1,475 @@
+"""Configuration, registry, weight reading and its errors, the cache's bookkeeping and the
+generation loop's decisions.  None of this needs a GPU."""
+
+import json
+import os
+import random
+
+import pytest
+import torch
+
+import fms_amd
+from fms_amd.architectures import list_models, list_variants, register_model, variant_config
+from fms_amd.cache import CacheFull, KVNeed, PagePool, SequenceCache, StateNeed
+from fms_amd.config import LLaMAConfig
+from fms_amd.engine.model import DecoderModel
+from fms_amd.architectures.llama import detect_source, llama_spec
+from fms_amd.generation import generate_requests, pad_input_ids, plan_batches, trim_prefix, truncate_after_eos
+from fms_amd.parts import ModelSpec, ScheduleEntry
+from fms_amd.weights import Checkpoint, WeightsError, get_adapter, kept_dtype, load_checkpoint, write_safetensors
+
+import plain_llama as P
+
+
+# --------------------------------------------------------------------------
+# configuration
+# --------------------------------------------------------------------------
+def test_config_defaults_and_derived_sizes():
+    c = LLaMAConfig()
+    assert (c.head_dim, c.kv_heads, c.ffn_hidden_dim) == (128, 32, 11008)
+    c = variant_config("llama", "3-8b")
+    assert (c.head_dim, c.kv_heads, c.ffn_hidden_dim, c.src_vocab_size) == (128, 8, 14336, 128256)
+    assert variant_config("llama", "3-70b").ffn_hidden_dim == 28672
+    assert LLaMAConfig(emb_dim=16, nheads=2, hidden_grow_factor=8 / 3, multiple_of=2).ffn_hidden_dim == 42
+
+
+def test_config_round_trip_and_updated(tmp_path):
+    c = LLaMAConfig(emb_dim=64, nheads=4, kvheads=2, rope_scaling={"rope_type": "llama3", "factor": 2.0})
+    path = tmp_path / "c.json"
+    c.save(path)
+    assert LLaMAConfig.load(path).as_dict() == c.as_dict()
+    # unknown keys in a file are dropped; updated() copies, does not touch the original, logs unknown names
+    data = c.as_dict()
+    data["never_heard_of"] = 1
+    path.write_text(json.dumps(data))
+    assert LLaMAConfig.load(path).as_dict() == c.as_dict()
+    d = c.updated(pad_id=5, bogus=1)
+    assert d.pad_id == 5 and c.pad_id == -1 and d is not c
+    d.rope_scaling["factor"] = 9.0
+    assert c.rope_scaling["factor"] == 2.0
+
+
+@pytest.mark.parametrize("bad", [dict(emb_dim=100, nheads=3), dict(nheads=4, kvheads=3), dict(emb_dim=12, nheads=4),
+                                 dict(activation_fn="gelu"), dict(rope_scaling={"rope_type": "yarn"})])
+def test_config_refuses_impossible_numbers(bad):
+    with pytest.raises(ValueError):
+        LLaMAConfig(**bad)
+
+
+def test_config_from_hugging_face_keys():
+    """The keys and the expected result of the reference's own mapping test
+    (tests/resources/fms_model_kwargs/tiny-LlamaForCausalLM-3.2.json)."""
+    hf = {"architectures": ["LlamaForCausalLM"], "hidden_size": 8, "intermediate_size": 32, "num_attention_heads": 4,
+          "num_key_value_heads": 2, "num_hidden_layers": 2, "rms_norm_eps": 1e-6, "rope_theta": 10000.0,
+          "vocab_size": 128256, "max_position_embeddings": 2048, "tie_word_embeddings": False,
+          "attention_bias": False, "mlp_bias": False, "hidden_act": "silu", "bos_token_id": 1, "torch_dtype": "float32"}
+    c = LLaMAConfig.from_hf_dict(hf)
+    expected = {"attn_bias": False, "emb_dim": 8, "hidden_grow_factor": 4.0, "kvheads": 2, "max_expected_seq_len": 2048,
+                "mlp_bias": False, "multiple_of": 1, "nheads": 4, "nlayers": 2, "norm_eps": 1e-06, "rope_theta": 10000.0,
+                "src_vocab_size": 128256, "tie_heads": False}
+    for k, v in expected.items():
+        assert getattr(c, k) == v, k
+    assert c.ffn_hidden_dim == 32
+    # the integer width survives ratios that int(ratio * width) would truncate
+    c = LLaMAConfig.from_hf_dict(dict(hf, hidden_size=440, num_attention_heads=4, intermediate_size=14336))
+    assert c.ffn_hidden_dim == 14336
+    assert LLaMAConfig.from_hf_dict(LLaMAConfig(emb_dim=64, nheads=4, kvheads=0).to_hf_dict()).kv_heads == 4
+    # rope parameters in the newer nesting; what the reference ignores silently is checked here
+    c = LLaMAConfig.from_hf_dict({**hf, "rope_parameters": {"rope_theta": 5e5, "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}}})
+    assert c.rope_theta == 5e5 and c.rope_scaling["rope_type"] == "llama3"
+    with pytest.raises(ValueError):
+        LLaMAConfig.from_hf_dict(dict(hf, head_dim=16))
+    with pytest.raises(ValueError):
+        LLaMAConfig.from_hf_dict(dict(hf, hidden_act="gelu"))
+    with pytest.raises(ValueError):
+        LLaMAConfig.from_hf_dict({k: v for k, v in hf.items() if k != "vocab_size"})
+
+
+def test_registry():
+    assert "llama" in list_models()
+    assert {"micro", "7b", "2-7b", "3-8b", "3-70b", "granite.code-8b"} <= set(list_variants("llama"))
+    with pytest.raises(KeyError):
+        register_model("llama", "micro", lambda **kw: LLaMAConfig())
+    with pytest.raises(KeyError):
+        list_variants("no_such_architecture")
+    with pytest.raises(KeyError):
+        variant_config("llama", "no_such_variant")
+    with pytest.raises(KeyError):
+        fms_amd.get_model("no_such_architecture", "x")
+    with pytest.raises(ValueError):
+        fms_amd.get_model("llama", "micro", data_type="int7")
+    assert variant_config("llama", "micro", nlayers=2).nlayers == 2
+    # a model folder's architecture comes from its config.json
+    from fms_amd.architectures import architecture_for_hf
+
+    assert architecture_for_hf("LlamaForCausalLM").name == "llama"
+    with pytest.raises(KeyError):
+        architecture_for_hf("GPTBigCodeForCausalLM")
+
+
+# --------------------------------------------------------------------------
+# weights
+# --------------------------------------------------------------------------
+TINY = dict(src_vocab_size=50, emb_dim=32, nheads=2, kvheads=1, nlayers=2, hidden_dim=40, multiple_of=1,
+            max_expected_seq_len=64)
+
+
+def test_model_declares_the_reference_tensor_names():
+    """tests/resources/expectations/models.test_llama.TestLlama2.test_model_weight_keys"""
+    model = DecoderModel(llama_spec(LLaMAConfig(**TINY)), torch.float32)
+    names = sorted(n for n, *_ in model.named_specs())
+    want = ["base_model.dec_norm.weight", "base_model.embedding.weight"]
+    for i in range(2):
+        p = f"base_model.layers.{i}."
+        want += [p + "attn.dense.weight", p + "attn.in_proj.qkv_fused.weight", p + "ff_ln.weight",
+                 p + "ff_sub_layer.w2.weight", p + "ff_sub_layer.wg1_fused.weight", p + "ln.weight"]
+    want.append("head.weight")
+    assert names == sorted(want)
+    biased = DecoderModel(llama_spec(LLaMAConfig(**TINY, attn_bias=True, mlp_bias=True)), torch.float32)
+    names = {n for n, *_ in biased.named_specs()}
+    assert "base_model.layers.0.attn.in_proj.qkv_fused.bias" in names and "base_model.layers.1.ff_sub_layer.w2.bias" in names
+
+
+def test_written_folder_is_read_back_the_same_by_both_readers(tmp_path):
+    config = LLaMAConfig(**TINY, tie_heads=True, attn_bias=True)
+    folder = fms_amd.write_model_folder(str(tmp_path / "m"), config, seed=3, norm_std=0.1)
+    again = fms_amd.write_model_folder(str(tmp_path / "m2"), config, seed=3, norm_std=0.1)
+    a = P.read_safetensors(os.path.join(folder, "model.safetensors"))
+    b = P.read_safetensors(os.path.join(again, "model.safetensors"))
+    assert a.keys() == b.keys() and all(torch.equal(a[k], b[k]) for k in a)  # a function of the seed
+    c = P.read_safetensors(os.path.join(fms_amd.write_model_folder(str(tmp_path / "m3"), config, seed=4), "model.safetensors"))
+    assert not torch.equal(a["model.embed_tokens.weight"], c["model.embed_tokens.weight"])
+    assert "lm_head.weight" not in a  # tied
+    assert a["model.layers.0.self_attn.q_proj.weight"].dtype == torch.bfloat16
+    # the product's reader and the installed safetensors package read the same values
+    ckpt = Checkpoint(folder, "hf")
+    from safetensors import safe_open
+
+    with safe_open(os.path.join(folder, "model.safetensors"), "pt") as f:
+        assert sorted(f.keys()) == sorted(ckpt.keys())
+        for k in f.keys():
+            assert torch.equal(f.get_tensor(k), ckpt.read(k))
+            assert torch.equal(a[k], ckpt.read(k))
+    ckpt.close()
+    from fms_amd.models import read_model_folder_config
+
+    arch, cfg = read_model_folder_config(folder)
+    assert arch.name == "llama" and cfg.ffn_hidden_dim == 40 and cfg.tie_heads and cfg.attn_bias
+
+
+def test_hf_adapter_matches_the_plain_conversion(tmp_path):
+    """Names, the row permutation of q/k (weights and biases) and the fusion order."""
+    config = LLaMAConfig(**TINY, attn_bias=True, mlp_bias=True)
+    folder = fms_amd.write_model_folder(str(tmp_path / "m"), config, seed=5)
+    cfg, want = P.load_model_folder(folder)
+    ckpt = Checkpoint(folder, "hf")
+    assert detect_source(ckpt.keys()) == "hf"
+    adapter = get_adapter("llama", "hf")
+    got = {}
+    from fms_amd.weights.loader import _layer_groups
+
+    for group in _layer_groups(ckpt.keys()):
+        got.update(adapter({n: ckpt.read(n) for n in group}, model_config=config))
+    ckpt.close()
+    assert sorted(got) == sorted(want)
+    for k in want:
+        assert torch.equal(got[k].float(), want[k]), k
+
+
+def test_meta_adapter_names_and_fusion():
+    """tests/utils/test_serialization.py:16-30: w1 is the gate, w3 the up projection, fused [w1; w3]."""
+    sd = {"layers.0.feed_forward.w1.weight": torch.ones(3, 2), "layers.0.feed_forward.w3.weight": torch.zeros(3, 2),
+          "layers.0.feed_forward.w2.weight": torch.ones(2, 3), "layers.0.attention.wq.weight": torch.full((4, 2), 1.0),
+          "layers.0.attention.wk.weight": torch.full((2, 2), 2.0), "layers.0.attention.wv.weight": torch.full((2, 2), 3.0),
+          "layers.0.attention.wo.weight": torch.ones(2, 4), "layers.0.attention_norm.weight": torch.ones(2),
+          "layers.0.ffn_norm.weight": torch.ones(2), "tok_embeddings.weight": torch.ones(5, 2),
+          "norm.weight": torch.ones(2), "output.weight": torch.ones(5, 2)}
+    assert detect_source(list(sd)) == "meta"
+    out = get_adapter("llama", "meta")(sd, model_config=None)
+    fused = out["base_model.layers.0.ff_sub_layer.wg1_fused.weight"]
+    assert torch.equal(fused, torch.cat([torch.ones(3, 2), torch.zeros(3, 2)]))
+    qkv = out["base_model.layers.0.attn.in_proj.qkv_fused.weight"]
+    assert qkv[:, 0].tolist() == [1, 1, 1, 1, 2, 2, 3, 3]
+    assert {"base_model.embedding.weight", "base_model.dec_norm.weight", "head.weight", "base_model.layers.0.ln.weight",
+            "base_model.layers.0.ff_ln.weight", "base_model.layers.0.attn.dense.weight",
+            "base_model.layers.0.ff_sub_layer.w2.weight"} <= set(out)
+    with pytest.raises(KeyError):
+        get_adapter("llama", "no_such_source")
+
+
+def test_kept_dtypes():
+    assert kept_dtype(torch.bfloat16, "float", torch.bfloat16) == torch.bfloat16
+    assert kept_dtype(torch.float16, "float", torch.bfloat16) == torch.bfloat16
+    assert kept_dtype(torch.float32, "float", torch.bfloat16) == torch.float32  # stored in 32-bit: stays so
+    assert kept_dtype(torch.bfloat16, "float", torch.float32) == torch.float32
+    assert kept_dtype(torch.int64, "int", torch.bfloat16) == torch.int32
+
+
+def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
+    config = LLaMAConfig(**TINY)
+    folder = fms_amd.write_model_folder(str(tmp_path / "m"), config, seed=1)
+    tensors = P.read_safetensors(os.path.join(folder, "model.safetensors"))
+    del tensors["model.layers.1.mlp.down_proj.weight"]
+    del tensors["model.norm.weight"]
+    tensors["model.layers.0.rotary_emb.inv_freq"] = torch.zeros(8)
+    tensors["model.layers.0.self_attn.o_proj.weight"] = torch.zeros(32, 48, dtype=torch.bfloat16)
+    write_safetensors(os.path.join(folder, "model.safetensors"), [(k, tuple(v.shape), v.dtype) for k, v in tensors.items()],
+                      lambda name: tensors[name])
+    model = DecoderModel(llama_spec(config), torch.float32, config=config)
+    with pytest.raises(WeightsError) as err:
+        load_checkpoint(model, folder, "llama", "hf", "cpu")
+    e = err.value
+    assert e.missing == ["base_model.dec_norm.weight", "base_model.layers.1.ff_sub_layer.w2.weight"]
+    assert e.unexpected == ["base_model.layers.0.rotary_emb.inv_freq"]
+    assert e.wrong_shapes == [("base_model.layers.0.attn.dense.weight", (32, 48), (32, 32))]
+    text = str(e)
+    for word in ("missing", "unexpected", "wrong shapes", "base_model.dec_norm.weight", "rotary_emb.inv_freq", "(32, 48)"):
+        assert word in text
+    with pytest.raises(FileNotFoundError, match="Can't find the requested checkpoint data at"):
+        Checkpoint(str(tmp_path / "nowhere"))
+
+
+def test_loading_keeps_types_and_ties_the_head(tmp_path):
+    config = LLaMAConfig(**TINY, tie_heads=True)
+    folder = fms_amd.write_model_folder(str(tmp_path / "m"), config, seed=2)
+    tensors = P.read_safetensors(os.path.join(folder, "model.safetensors"))
+    tensors["model.norm.weight"] = tensors["model.norm.weight"].float()  # one tensor stored in 32-bit
+    write_safetensors(os.path.join(folder, "model.safetensors"), [(k, tuple(v.shape), v.dtype) for k, v in tensors.items()],
+                      lambda name: tensors[name])
+    model = DecoderModel(llama_spec(config), torch.bfloat16, config=config)
+    load_checkpoint(model, folder, "llama", "hf", "cpu")
+    assert model.final_norm.w["weight"].dtype == torch.float32
+    assert model.layers[0].mixer.qkv.w["weight"].dtype == torch.bfloat16
+    assert model.head.w["weight"] is model.embedding.w["weight"]
+    model32 = DecoderModel(llama_spec(config), torch.float32, config=config)
+    load_checkpoint(model32, folder, "llama", "hf", "cpu")
+    assert model32.layers[1].feed_forward.w2.w["weight"].dtype == torch.float32
+
+
+def test_schedule_is_data():
+    config = LLaMAConfig(**TINY)
+    spec = llama_spec(config)
+    spec.schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0), ScheduleEntry(1, cache_of=1)]
+    model = DecoderModel(spec, torch.float32)
+    kv, state = model.cache_needs()
+    assert [e for e, _ in kv] == [0, 1, 2] and state == []  # entry 3 reads entry 1's cache
+    cache = model.make_cache(256, 2, device=None)
+    assert len(cache.groups) == 1 and cache.groups[0].entries == [0, 1, 2]
+    for bad in ([ScheduleEntry(5)], [ScheduleEntry(0, cache_of=0)], [ScheduleEntry(0), ScheduleEntry(1, cache_of=1)]):
+        spec.schedule = bad
+        with pytest.raises(ValueError):
+            DecoderModel(spec, torch.float32)
+
+
+# --------------------------------------------------------------------------
+# cache
+# --------------------------------------------------------------------------
+def test_page_pool_accounting():
+    pool = PagePool(3)
+    pages = [pool.alloc() for _ in range(3)]
+    assert sorted(pages) == [0, 1, 2] and pool.n_free == 0
+    with pytest.raises(CacheFull):
+        pool.alloc()
+    pool.free(pages[1])
+    with pytest.raises(ValueError):
+        pool.free(pages[1])  # freed twice
+    with pytest.raises(ValueError):
+        pool.free(7)
+    assert pool.alloc() == pages[1]
+    pool.check()
+
+
+def make_cache(max_tokens=64 * 6, max_slots=3, window=0):
+    needs = [(0, KVNeed(2, 16)), (1, KVNeed(2, 16)), (2, KVNeed(2, 16, window))] if window else [(0, KVNeed(2, 16)), (1, KVNeed(2, 16))]
+    return SequenceCache(needs, [(1, StateNeed((("sum", (4,), "float32"),)))], max_tokens, max_slots, 1000)
+
+
+def test_cache_slots_and_pages_never_leak():
+    cache = make_cache()
+    rng = random.Random(0)
+    live = {}
+    for _ in range(2000):
+        action = rng.random()
+        if action < 0.3 and cache.n_free_slots:
+            s = cache.alloc_slot()
+            assert s not in live
+            live[s] = 0
+        elif action < 0.8 and live:
+            s = rng.choice(list(live))
+            n = rng.choice([1, 1, 1, 5, 64, 70])
+            try:
+                start = cache.extend(s, n)
+                assert start == live[s]
+                live[s] += n
+            except CacheFull:
+                assert cache.length(s) == live[s]  # nothing changed
+        elif live:
+            s = rng.choice(list(live))
+            cache.free_slot(s)
+            del live[s]
+            with pytest.raises(ValueError):
+                cache.free_slot(s)  # freed twice
+        cache.check()
+        held = sum(-(-n // 64) for n in live.values())
+        assert cache.groups[0].pool.n_held == held
+    for s in list(live):
+        cache.free_slot(s)
+    cache.check()
+    assert cache.groups[0].pool.n_free == 6 and cache.n_free_slots == 3
+    with pytest.raises(CacheFull):
+        [cache.alloc_slot() for _ in range(4)]
+
+
+def test_cache_groups_and_window_pages():
+    cache = make_cache(max_tokens=64 * 8, window=100)
+    assert len(cache.groups) == 2 and cache.groups[0].entries == [0, 1] and cache.groups[1].entries == [2]
+    s = cache.alloc_slot()
+    cache.extend(s, 300)
+    assert len(cache.groups[0].pages[s]) == 5 and cache.groups[1].pool.n_held == 5
+    for _ in range(100):
+        cache.extend(s, 1)  # decoding: the windowed group gives back pages no later query can see
+    cache.check()
+    assert cache.groups[0].pool.n_held == 7
+    # position 399 sees keys >= 300: logical pages 0..3 are gone
+    table = cache.block_table(1, [s])
+    assert (table[0, :4] == -1).all() and (table[0, 4:7] >= 0).all()
+    assert cache.groups[1].pool.n_held == 3
+    with pytest.raises(IndexError):
+        cache.extend(s, 1000)  # beyond the model's positions
+    cache.free_slot(s)
+    cache.check()
+    assert cache.groups[1].pool.n_free == 8
+
+
+def test_block_table_rows_follow_the_step_order():
+    cache = make_cache()
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    cache.extend(a, 65)
+    cache.extend(b, 3)
+    table = cache.block_table(0, [b, a])
+    assert table.shape == (2, 2) and table[0, 1] == -1 and table[1, 1] >= 0
+    assert set(table.flatten().tolist()) - {-1} == set(cache.groups[0].pages[a] + cache.groups[0].pages[b])
+
+
+# --------------------------------------------------------------------------
+# generation loop
+# --------------------------------------------------------------------------
+class FakeEngine:
+    """Next token = last token + 1 (the mock of tests/utils/test_generate.py:15-30), with a real cache's bookkeeping."""
+
+    class _Cache:
+        pass
+
+    def __init__(self, max_tokens=64 * 8, max_slots=4, max_seq_len=100, vocab=256):
+        self.cache = SequenceCache([(0, KVNeed(1, 2))], [], max_tokens, max_slots, max_seq_len)
+        self.vocab = vocab
+        self.device = torch.device("cpu")
+        self.steps = []
+        self.last = {}
+
+    def new_sequence(self):
+        return self.cache.alloc_slot()
+
+    def end_sequence(self, slot):
+        self.cache.free_slot(slot)
+        self.cache.check()
+
+    def step(self, slots, tokens, want):
+        assert want == "last"
+        self.steps.append([len(t) for t in tokens])
+        logits = torch.zeros(len(slots), self.vocab)
+        for i, (s, t) in enumerate(zip(slots, tokens)):
+            self.cache.extend(s, len(t))
+            logits[i, (t[-1] + 1) % self.vocab] = 1.0
+        return logits
+
+
+def argmax_chooser(logits, request_ids, counters):
+    return logits.argmax(-1).tolist()
+
+
+def test_loop_counts_up_like_the_reference_mock():
+    """tests/utils/test_generate.py:33-50: "ABCDE" -> "ABCDEFGHIJ"."""
+    engine = FakeEngine()
+    out = generate_requests(engine, [[ord(c) for c in "ABCDE"]], max_new_tokens=5, chooser=argmax_chooser)
+    assert "".join(chr(t) for t in out[0]) == "FGHIJ"
+    assert engine.steps == [[5], [1], [1], [1], [1]]  # the prompt in one step, then one token each
+    assert engine.cache.live_slots() == []
+
+
+def test_loop_unequal_prompts_stops_and_limits():
+    engine = FakeEngine()
+    prompts = [[10, 11, 12], [50], [20, 21], [97, 98]]
+    out = generate_requests(engine, prompts, max_new_tokens=6, stop_token_ids=[23, 52], chooser=argmax_chooser)
+    assert out == [[13, 14, 15, 16, 17, 18], [51, 52], [22, 23], [99, 100, 101, 102, 103, 104]]
+    # the batch shrinks as sequences end: 4 prompts, 4 alive, then 2
+    assert engine.steps == [[3, 1, 2, 2], [1, 1, 1, 1], [1, 1], [1, 1], [1, 1], [1, 1]]
+    # a sequence stops at the model's last position: prompt 2 + 98 new = 100 tokens, the last one is not fed
+    engine = FakeEngine(max_seq_len=100, max_tokens=64 * 4)
+    out = generate_requests(engine, [[1, 2]], max_new_tokens=500, chooser=argmax_chooser)
+    assert len(out[0]) == 99 and engine.cache.live_slots() == []
+    assert generate_requests(engine, [[1]], max_new_tokens=0, chooser=argmax_chooser) == [[]]
+
+
+def test_loop_runs_as_many_batches_as_the_requests_need():
+    engine = FakeEngine(max_tokens=64 * 2, max_slots=2)
+    prompts = [[i] for i in range(7)]
+    out = generate_requests(engine, prompts, max_new_tokens=3, chooser=argmax_chooser)
+    assert out == [[i + 1, i + 2, i + 3] for i in range(7)]
+    assert engine.steps[0] == [1, 1] and len([s for s in engine.steps if s == [1]]) == 3  # 3 full batches and a last one of 1
+    assert plan_batches([5, 70, 10, 200], 60, 64 * 6, 3, 1000) == [[0, 1], [2], [3]]
+    assert plan_batches([5, 70, 10, 100], 60, 64 * 6, 3, 1000) == [[0, 1], [2, 3]]
+    assert plan_batches([1, 1, 1], 1, 64 * 8, 2, 1000) == [[0, 1], [2]]
+    with pytest.raises(ValueError):
+        plan_batches([500], 10, 64 * 4, 2, 1000)
+    with pytest.raises(IndexError):
+        plan_batches([50], 10, 64 * 4, 2, 40)
+    with pytest.raises(ValueError):
+        plan_batches([0], 10, 64 * 4, 2, 40)
+    # a failing step gives its slots back
+    class Broken(FakeEngine):
+        def step(self, *a):
+            raise RuntimeError("boom")
+
+    engine = Broken()
+    with pytest.raises(RuntimeError):
+        generate_requests(engine, [[1], [2]], max_new_tokens=3, chooser=argmax_chooser)
+    assert engine.cache.live_slots() == []
+
+
+def test_padding_helpers_follow_the_reference():
+    """tests/utils/test_generate.py:148-198: exact tensors of pad_input_ids."""
+    ids, extra = pad_input_ids([torch.arange(1, 5), torch.arange(1, 8)])
+    assert ids.tolist() == [[0, 0, 0, 1, 2, 3, 4], [1, 2, 3, 4, 5, 6, 7]]
+    assert extra["position_ids"].tolist() == [[0, 0, 0, 0, 1, 2, 3], [0, 1, 2, 3, 4, 5, 6]]
+    m = extra["mask"][0]
+    assert m[3, 3] == 0 and m[3, 2] == -torch.inf and m[6, 3] == 0 and m[6, 0] == -torch.inf and m[1, 0] == 0 and m[0, 1] == -torch.inf
+    assert extra["lengths"] == [4, 7]
+    # tests/utils/test_generate.py:139-145 and :281-286
+    assert truncate_after_eos(torch.tensor([5, 6, 3, 9, 3]), 3).tolist() == [5, 6, 3]
+    assert truncate_after_eos(torch.tensor([5, 6]), None).tolist() == [5, 6]
+    assert trim_prefix(torch.tensor([0, 0, 0, 0, 1, 2, 3, 4])).tolist() == [1, 2, 3, 4]
+    assert trim_prefix(torch.tensor([0, 0, 0, 0, 1, 2, 3, 4]), 5).tolist() == [0, 0, 0, 0, 1, 2, 3, 4]
+    assert trim_prefix(torch.tensor([1, 2, 3, 4, 0, 1])).tolist() == [1, 2, 3, 4, 0, 1]
+
+
+def test_sampling_uniforms_are_a_function_of_seed_and_counter():
+    from fms_amd.sampling import SamplingParams, request_seed, uniform
+
+    us = [uniform(request_seed(3, r), c) for r in range(4) for c in range(50)]
+    assert all(0 <= u < 1 for u in us) and len(set(us)) > 190
+    assert 0.35 < sum(us) / len(us) < 0.65
+    assert uniform(5, 9) == uniform(5, 9) and uniform(5, 9) != uniform(5, 10) != uniform(6, 9)
+    with pytest.raises(ValueError):
+        SamplingParams(do_sample=True, temperature=0.0)
+
+
+def test_no_gpu_means_a_loud_failure():
+    if torch.cuda.is_available():
+        pytest.skip("this machine has a GPU")
+    with pytest.raises(RuntimeError):
+        fms_amd.get_model("llama", "micro", device_type="cpu")
+    from fms_amd.kernels import ops
+
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4))

@@ -1,0 +1,256 @@
+"""Pins of the plain implementation: what fixes it beside the reference's text.
+
+* the output signatures the reference's own tests store
+  (tests/resources/expectations/models.test_llama.*.test_model_output),
+* special cases that reduce to a library routine,
+* invariants chosen so that a plausible mistake fails them.
+"""
+
+import math
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+import plain_llama as P
+
+# The four stored signatures (16 floats each), copied from the reference's
+# tests/resources/expectations/models.test_llama.<Class>.test_model_output
+SIGNATURES = {
+    "TestLlama2": "0.052729345858097076,0.011515989899635315,0.007392197847366333,0.0,0.01378333568572998,0.012065891176462173,0.03835539519786835,0.02802693098783493,0.020719021558761597,0.027966909110546112,0.014432244002819061,0.03975895047187805,0.05111371725797653,0.04628599435091019,0.0315752848982811,0.01688060164451599",
+    "TestLlama2GQA": "0.033434536308050156,0.03998075798153877,0.020981933921575546,0.0,0.040768157690763474,0.03792032226920128,0.026382219046354294,0.033903587609529495,0.012676555663347244,0.0020506493747234344,0.026054974645376205,0.003850828856229782,0.033241596072912216,0.006034858524799347,0.004931684583425522,0.022256117314100266",
+    "TestLlama3": "0.03351592645049095,0.040137480944395065,0.021625619381666183,0.0,0.03257865831255913,0.036533039063215256,0.027063172310590744,0.037584420293569565,0.01366950199007988,0.002703893929719925,0.025658320635557175,0.0047348253428936005,0.03350717946887016,0.0010565221309661865,0.007586400955915451,0.02299729362130165",
+    "TestLlama31": "0.03351592645049095,0.040137480944395065,0.021625619381666183,0.0,0.03257865831255913,0.036533039063215256,0.027063172310590744,0.03758440539240837,0.01366950199007988,0.002703893929719925,0.025658313184976578,0.0047348253428936005,0.03350717946887016,0.0010565221309661865,0.007586400955915451,0.02299729362130165",
+}
+
+# configurations of those tests: tests/models/test_llama.py:30-45, :108-122, :196-211 and :232-253
+SIG_CONFIGS = {
+    "TestLlama2": dict(seed=0, nheads=2, kvheads=2, grow=8 / 3, theta=10000.0, max_len=4096, scaling={}),
+    "TestLlama2GQA": dict(seed=5, nheads=4, kvheads=2, grow=8 / 3, theta=10000.0, max_len=4096, scaling={}),
+    "TestLlama3": dict(seed=5, nheads=4, kvheads=2, grow=3.5, theta=500000.0, max_len=8192, scaling={}),
+    "TestLlama31": dict(
+        seed=5,
+        nheads=4,
+        kvheads=2,
+        grow=3.5,
+        theta=500000.0,
+        max_len=131072,
+        scaling={
+            "factor": 8.0,
+            "low_freq_factor": 1.0,
+            "high_freq_factor": 4.0,
+            "original_max_position_embeddings": 8192,
+            "rope_type": "llama3",
+        },
+    ),
+}
+
+
+def _fixture_weights(cfg: P.PlainConfig, seed: int):
+    """fms/testing/_internal/model_test_suite.py:61-79: every tensor of the state dict,
+    in sorted-name order, is (randn - 0.5) / 20 under one seed."""
+    D = cfg.head_dim
+    shapes = {
+        "base_model.dec_norm.weight": (cfg.width,),
+        "base_model.embedding.weight": (cfg.vocab, cfg.width),
+        "head.weight": (cfg.vocab, cfg.width),
+    }
+    for i in range(cfg.nlayers):
+        p = f"base_model.layers.{i}."
+        shapes[p + "attn.dense.weight"] = (cfg.width, cfg.nheads * D)
+        shapes[p + "attn.in_proj.qkv_fused.weight"] = ((cfg.nheads + 2 * cfg.kvheads) * D, cfg.width)
+        shapes[p + "ff_ln.weight"] = (cfg.width,)
+        shapes[p + "ff_sub_layer.w2.weight"] = (cfg.width, cfg.hidden)
+        shapes[p + "ff_sub_layer.wg1_fused.weight"] = (2 * cfg.hidden, cfg.width)
+        shapes[p + "ln.weight"] = (cfg.width,)
+    torch.random.manual_seed(seed)
+    weights = {}
+    for name in sorted(shapes):
+        values = torch.randn(shapes[name])
+        values -= 0.5
+        values /= 20.0
+        weights[name] = values
+    return weights
+
+
+@pytest.mark.parametrize("name", sorted(SIGNATURES))
+def test_reference_signature(name):
+    c = SIG_CONFIGS[name]
+    cfg = P.PlainConfig(
+        vocab=381,
+        width=16,
+        nheads=c["nheads"],
+        kvheads=c["kvheads"],
+        nlayers=2,
+        hidden=P.glu_hidden(16, c["grow"], 2),
+        eps=1e-5,
+        theta=c["theta"],
+        max_len=c["max_len"],
+        rope_scaling=c["scaling"],
+    )
+    weights = _fixture_weights(cfg, c["seed"])
+    logits = P.forward(weights, cfg, list(range(16)))
+    # fms/testing/comparison.py:104-105
+    s = logits.max(-1).values - logits.min(-1).values
+    signature = s - s.min()
+    expected = torch.tensor([float(v) for v in SIGNATURES[name].split(",")])
+    torch.testing.assert_close(signature, expected)
+
+
+def test_glu_hidden_sizes():
+    assert P.glu_hidden(16, 8 / 3, 2) == 42
+    assert P.glu_hidden(4096, 8 / 3, 256) == 11008
+    assert P.glu_hidden(4096, 3.5, 1024) == 14336
+    assert P.glu_hidden(8192, 1.3 * 8 / 3, 4096) == 28672
+
+
+def test_rms_norm_is_library_rms_norm():
+    torch.manual_seed(1)
+    x = torch.randn(5, 24) * 3
+    w = torch.randn(24)
+    torch.testing.assert_close(P.rms_norm(x, w, 1e-3), F.rms_norm(x, (24,), w, 1e-3))
+    # eps inside the root: a zero row gives zeros, not NaN
+    assert torch.equal(P.rms_norm(torch.zeros(1, 24), w, 1e-5), torch.zeros(1, 24))
+    # a large eps visibly shrinks the output (eps outside the root or forgotten would not)
+    y = P.rms_norm(torch.ones(1, 4), torch.ones(4), 3.0)
+    torch.testing.assert_close(y, torch.full((1, 4), 0.5))
+
+
+def test_rope_reference_vectors():
+    """tests/modules/test_positions.py:47-72: D=2, theta=1 rotates by `pos` radians."""
+    x = torch.tensor([[1.0, 0.0], [1.0, 0.0]]).reshape(2, 1, 2)
+    out = P.rope_rotate(x, torch.arange(2), P.rope_frequencies(2, 1.0))
+    torch.testing.assert_close(out[0, 0], torch.tensor([1.0, 0.0]))
+    torch.testing.assert_close(out[1, 0], torch.tensor([math.cos(1.0), math.sin(1.0)]))
+
+
+def test_rope_is_complex_multiplication():
+    torch.manual_seed(2)
+    D = 24
+    x = torch.randn(7, 3, D)
+    pos = torch.tensor([0, 1, 2, 5, 9, 100, 1000])
+    freqs = P.rope_frequencies(D, 500000.0)
+    out = P.rope_rotate(x, pos, freqs)
+    z = torch.view_as_complex(x.reshape(7, 3, D // 2, 2).contiguous())
+    rot = torch.polar(torch.ones(7, D // 2), torch.outer(pos.float(), freqs))[:, None, :]
+    torch.testing.assert_close(out, torch.view_as_real(z * rot).reshape(7, 3, D))
+    # position 0 is the identity; norms are kept
+    torch.testing.assert_close(out[0], x[0])
+    torch.testing.assert_close(out.norm(dim=-1), x.norm(dim=-1))
+
+
+def test_rope_scores_depend_on_distance_only():
+    """tests/modules/test_positions.py:191-214: a shift of all positions changes no score."""
+    torch.manual_seed(3)
+    D = 16
+    q = torch.randn(6, 1, D)
+    k = torch.randn(6, 1, D)
+    freqs = P.rope_frequencies(D, 10000.0)
+    pos = torch.arange(6)
+    s0 = P.rope_rotate(q, pos, freqs)[:, 0] @ P.rope_rotate(k, pos, freqs)[:, 0].t()
+    s1 = P.rope_rotate(q, pos + 37, freqs)[:, 0] @ P.rope_rotate(k, pos + 37, freqs)[:, 0].t()
+    torch.testing.assert_close(s0, s1, atol=1e-4, rtol=1e-4)
+    # ...and a wrong sign of the sine would still pass the above, so pin the direction:
+    one = P.rope_rotate(torch.tensor([1.0, 0.0]).reshape(1, 1, 2), torch.tensor([1]), torch.tensor([0.5]))
+    assert one[0, 0, 1] > 0
+
+
+def test_rope_pairings_agree_after_row_permutation():
+    """fms/models/llama.py:711-721: half-split rotation of HF-ordered rows equals
+    adjacent-pair rotation of the permuted rows, up to the same permutation of the output."""
+    torch.manual_seed(4)
+    D, heads, E, S = 16, 3, 10, 5
+    w_hf = torch.randn(heads * D, E)
+    x = torch.randn(S, E)
+    pos = torch.arange(S) + 3
+    freqs = P.rope_frequencies(D, 10000.0)
+    q_hf = P.rope_rotate_halves((x @ w_hf.t()).reshape(S, heads, D), pos, freqs)
+    q_ref = P.rope_rotate((x @ P._halves_to_pairs(w_hf, D).t()).reshape(S, heads, D), pos, freqs)
+    # scores are what matters: a dot product over the head is permutation invariant
+    torch.testing.assert_close(
+        torch.einsum("shd,thd->hst", q_hf, q_hf), torch.einsum("shd,thd->hst", q_ref, q_ref), atol=1e-4, rtol=1e-4
+    )
+    # and element-wise: reference element 2i+j is HF element j*D/2+i
+    torch.testing.assert_close(q_ref.reshape(S, heads, D // 2, 2).transpose(2, 3).reshape(S, heads, D), q_hf)
+
+
+def test_rope_llama3_scaling_limits():
+    scaling = {
+        "rope_type": "llama3",
+        "factor": 8.0,
+        "low_freq_factor": 1.0,
+        "high_freq_factor": 4.0,
+        "original_max_position_embeddings": 8192,
+    }
+    base = P.rope_frequencies(128, 500000.0)
+    scaled = P.rope_frequencies(128, 500000.0, scaling)
+    wavelen = 2 * math.pi / base
+    assert torch.equal(scaled[wavelen < 8192 / 4], base[wavelen < 8192 / 4])
+    torch.testing.assert_close(scaled[wavelen > 8192], base[wavelen > 8192] / 8)
+    mid = (wavelen >= 8192 / 4) & (wavelen <= 8192)
+    assert mid.any() and bool(((scaled[mid] < base[mid]) & (scaled[mid] > base[mid] / 8)).all())
+
+
+@pytest.mark.parametrize("H,K", [(4, 4), (4, 2), (4, 1), (1, 1)])
+def test_attention_is_library_attention(H, K):
+    torch.manual_seed(5)
+    S, D = 9, 8
+    q, k, v = torch.randn(S, H, D), torch.randn(S, K, D), torch.randn(S, K, D)
+    ours = P.causal_attention(q, k, v)
+    ke = k.repeat_interleave(H // K, dim=1)
+    ve = v.repeat_interleave(H // K, dim=1)
+    lib = F.scaled_dot_product_attention(
+        q.transpose(0, 1)[None], ke.transpose(0, 1)[None], ve.transpose(0, 1)[None], is_causal=True
+    )[0].transpose(0, 1)
+    torch.testing.assert_close(ours, lib, atol=1e-5, rtol=1e-5)
+
+
+def test_attention_special_cases():
+    torch.manual_seed(6)
+    S, H, K, D = 6, 4, 2, 8
+    q, k, v = torch.randn(S, H, D), torch.randn(S, K, D), torch.randn(S, K, D)
+    out = P.causal_attention(q, k, v)
+    # the first query sees one key: its output is that key's value, of its own kv head
+    torch.testing.assert_close(out[0, 0], v[0, 0])
+    torch.testing.assert_close(out[0, 3], v[0, 1])
+    # zero queries average the visible values
+    avg = P.causal_attention(torch.zeros_like(q), k, v)
+    torch.testing.assert_close(avg[3, 2], v[:4, 1].mean(0))
+    # a window of 1 sees only the token itself
+    win = P.causal_attention(q, k, v, window=1)
+    torch.testing.assert_close(win[:, 1], v[:, 0])
+
+
+def test_feed_forward_gate_comes_first():
+    """tests/utils/test_fusion.py:28-41, tests/utils/test_serialization.py:16-25: fused = [gate; up]."""
+    torch.manual_seed(7)
+    E, Fh = 6, 10
+    wg, w1, w2 = torch.randn(Fh, E), torch.randn(Fh, E), torch.randn(E, Fh)
+    x = torch.randn(4, E)
+    fused = P.gated_feed_forward(x, torch.cat([wg, w1]), w2)
+    torch.testing.assert_close(fused, (F.silu(x @ wg.t()) * (x @ w1.t())) @ w2.t())
+    # a zero gate gives zero, a zero "up" too; swapping the halves would change this
+    zero_gate = P.gated_feed_forward(x, torch.cat([torch.zeros(Fh, E), w1]), w2)
+    assert torch.equal(zero_gate, torch.zeros(4, E))
+
+
+def test_forward_prefix_property():
+    """Causality: logits of a prefix do not change when tokens are appended."""
+    cfg = P.PlainConfig(vocab=50, width=24, nheads=3, kvheads=1, nlayers=2, hidden=40, eps=1e-5, theta=1e4, max_len=64)
+    weights = _fixture_weights(cfg, 11)
+    ids = [3, 9, 4, 4, 17, 30, 2, 8]
+    full = P.forward(weights, cfg, ids)
+    part = P.forward(weights, cfg, ids[:5])
+    torch.testing.assert_close(full[:5], part, atol=1e-5, rtol=1e-5)
+    with pytest.raises(IndexError):
+        P.forward(weights, cfg, list(range(40)), first_position=30)
+
+
+def test_sampling_distribution():
+    logits = torch.tensor([1.0, 3.0, 2.0, 3.0, -1.0])
+    p = P.sampling_distribution(logits, 0.5, 2)
+    # ties at the threshold survive (fms/utils/generation.py:322-323)
+    torch.testing.assert_close(p, torch.tensor([0.0, 0.5, 0.0, 0.5, 0.0]))
+    p = P.sampling_distribution(logits, 2.0, 0)
+    torch.testing.assert_close(p, torch.softmax(logits / 2.0, -1))
+    assert P.greedy(torch.tensor([0.1, 0.7, 0.3])) == 1
