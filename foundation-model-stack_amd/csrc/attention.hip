@@ -210,23 +210,23 @@ __device__ __forceinline__ void load_query(bf16x8 (&dst)[(MAXDT + 1) / 2], const
 }
 
 // ==========================================================================
-// prefill: a block is PREFILL_WAVES waves, each with 16*QT consecutive query
+// prefill: a block is WAVES waves, each with 16*QT consecutive query
 // tokens of one sequence, for one query head.  Keys come from the cache, so a
 // chunk that continues a cached prefix works the same way.
 // ==========================================================================
-#define PREFILL_WAVES 4
-#define PREFILL_QT 2
-#define PREFILL_QBLOCK (PREFILL_WAVES * PREFILL_QT * 16)
+// A block covers PREFILL_QBLOCK tokens as WAVES waves of 16*QT tokens; large head sizes take
+// fewer tokens per wave so that the accumulators stay in registers.
+#define PREFILL_QBLOCK 128
 
-template <int MAXDT>
-__global__ void __launch_bounds__(PREFILL_WAVES* WAVE)
+template <int MAXDT, int QT, int WAVES>
+__global__ void __launch_bounds__(WAVES* WAVE)
     attn_prefill_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                              const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                              const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                              const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                              const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
                              int window) {
-  constexpr int QT = PREFILL_QT;
+  static_assert(WAVES * QT * 16 == PREFILL_QBLOCK, "a block covers PREFILL_QBLOCK tokens");
   const int h = blockIdx.y;
   const int wave = threadIdx.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
@@ -470,17 +470,16 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
   FMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attn_prefill_bf16: row strides must keep 16-byte alignment");
   FMS_REQUIRE(nheads <= 65535, "attn_prefill_bf16: too many heads");
   dim3 grid(n_qblocks, nheads);
-  dim3 block(PREFILL_WAVES * WAVE);
-#define FMS_PF(M)                                                                                                   \
-  attn_prefill_bf16_kernel<M><<<grid, block, 0, stream>>>(                                                          \
+#define FMS_PF(M, QT, WAVES)                                                                                        \
+  attn_prefill_bf16_kernel<M, QT, WAVES><<<grid, dim3(WAVES * WAVE), 0, stream>>>(                                  \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window)
   if (head_dim <= 64)
-    FMS_PF(4);
+    FMS_PF(4, 2, 4);
   else if (head_dim <= 128)
-    FMS_PF(8);
+    FMS_PF(8, 2, 4);
   else
-    FMS_PF(16);
+    FMS_PF(16, 1, 8);
 #undef FMS_PF
   FMS_LAUNCH_CHECK("attn_prefill_bf16");
   return 0;

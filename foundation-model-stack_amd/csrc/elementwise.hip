@@ -60,7 +60,7 @@ extern "C" int fmsamd_embed(const int* ids, const void* table, int table_dtype, 
 // residual is not written back (the stream is not used again).
 // --------------------------------------------------------------------------
 template <typename BranchT, typename WeightT, typename OutT>
-__global__ void add_norm_kernel(float* __restrict__ resid, const BranchT* __restrict__ branch,
+__global__ void __launch_bounds__(1024) add_norm_kernel(float* __restrict__ resid, const BranchT* __restrict__ branch,
                                 const WeightT* __restrict__ weight, const WeightT* __restrict__ bias,
                                 OutT* __restrict__ out, const int* __restrict__ rows, int width, float eps,
                                 int use_mean) {
@@ -70,37 +70,66 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const BranchT* __rest
   const BranchT* b = branch ? branch + (size_t)r * width : nullptr;
   OutT* o = out + (size_t)blockIdx.x * width;
 
-  constexpr int KEEP = 16;  // values a thread keeps in registers; wider rows are read again
+  // The first KEEP values of a thread stay in registers; a wider row is read again.  The loops over
+  // the kept values have compile-time trip counts: the array must never be indexed by a run-time
+  // value, or it is addressed through relative register indexing.
+  constexpr int KEEP = 16;
   float keep[KEEP];
+  const int tail = threadIdx.x + KEEP * blockDim.x;
   float sum = 0.f, sq = 0.f;
-  int n = 0;
-  for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * blockDim.x;
+    float v = 0.f;
+    if (i < width) {
+      v = x[i];
+      if (b) {
+        v += to_f32(b[i]);
+        if (!rows) x[i] = v;
+      }
+    }
+    keep[n] = v;
+    sum += v;
+    sq += v * v;
+  }
+  for (int i = tail; i < width; i += blockDim.x) {
     float v = x[i];
     if (b) {
       v += to_f32(b[i]);
       if (!rows) x[i] = v;
     }
-    if (n < KEEP) keep[n] = v;
     sum += v;
     sq += v * v;
   }
+  const bool reread_adds = rows != nullptr && b != nullptr;  // the stream was not updated: add again
   float mean = 0.f;
   if (use_mean) {
     mean = block_sum(sum, scratch) / (float)width;
-    // second moment about the mean, from the kept values
-    sq = 0.f;
-    n = 0;
-    for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
-      float v = (n < KEEP ? keep[n] : (rows && b ? x[i] + to_f32(b[i]) : x[i])) - mean;
+    sq = 0.f;  // second moment about the mean
+#pragma unroll
+    for (int n = 0; n < KEEP; ++n) {
+      const int i = threadIdx.x + n * blockDim.x;
+      if (i < width) sq += (keep[n] - mean) * (keep[n] - mean);
+    }
+    for (int i = tail; i < width; i += blockDim.x) {
+      const float v = (reread_adds ? x[i] + to_f32(b[i]) : x[i]) - mean;
       sq += v * v;
     }
   }
   const float ms = block_sum(sq, scratch) / (float)width;
   const float scale = rsqrtf(ms + eps);
-  n = 0;
-  for (int i = threadIdx.x; i < width; i += blockDim.x, ++n) {
-    float v = n < KEEP ? keep[n] : (rows && b ? x[i] + to_f32(b[i]) : x[i]);
-    v = (v - mean) * scale;
+#pragma unroll
+  for (int n = 0; n < KEEP; ++n) {
+    const int i = threadIdx.x + n * blockDim.x;
+    if (i < width) {
+      float v = (keep[n] - mean) * scale;
+      if (weight) v *= to_f32(weight[i]);
+      if (bias) v += to_f32(bias[i]);
+      o[i] = from_f32<OutT>(v);
+    }
+  }
+  for (int i = tail; i < width; i += blockDim.x) {
+    float v = ((reread_adds ? x[i] + to_f32(b[i]) : x[i]) - mean) * scale;
     if (weight) v *= to_f32(weight[i]);
     if (bias) v += to_f32(bias[i]);
     o[i] = from_f32<OutT>(v);
@@ -110,7 +139,7 @@ __global__ void add_norm_kernel(float* __restrict__ resid, const BranchT* __rest
 template <typename BranchT, typename WeightT, typename OutT>
 static void launch_add_norm(float* resid, const void* branch, const void* weight, const void* bias, void* out,
                             const int* rows, int n_out, int width, float eps, int use_mean, hipStream_t stream) {
-  const int threads = width >= 2048 ? 256 : (width >= 512 ? 128 : 64);
+  const int threads = width > 4096 ? 1024 : (width >= 2048 ? 256 : (width >= 512 ? 128 : 64));
   add_norm_kernel<BranchT, WeightT, OutT><<<n_out, threads, 0, stream>>>(
       resid, (const BranchT*)branch, (const WeightT*)weight, (const WeightT*)bias, (OutT*)out, rows, width, eps,
       use_mean);

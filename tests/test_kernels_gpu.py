@@ -41,7 +41,7 @@ def test_embed(ops):
         assert torch.equal(out, table.float()[ids.long()])
 
 
-@pytest.mark.parametrize("width", [24, 100, 4096, 9000])
+@pytest.mark.parametrize("width", [24, 100, 4096, 9000, 20000])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_add_norm(ops, width, dtype):
     torch.manual_seed(1)

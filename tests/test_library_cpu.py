@@ -473,3 +473,31 @@ def test_no_gpu_means_a_loud_failure():
 
     with pytest.raises(RuntimeError, match="no CPU fallback"):
         ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4))
+
+
+# --------------------------------------------------------------------------
+# the compiled kernels
+# --------------------------------------------------------------------------
+def test_kernels_compile_without_relative_register_indexing(tmp_path):
+    """A private array indexed by a run-time value is addressed through relative register
+    indexing (s_set_gpr_idx / v_movrel); the compiler may then write the indexed register
+    unconditionally and select afterwards, and an index past the array lands in a live
+    register of the same wave.  No kernel here may need that, nor spill registers."""
+    import re
+    import subprocess
+
+    import importlib
+
+    build = importlib.import_module("fms_amd.kernels.build")
+    try:
+        hipcc = build.hipcc_path()
+    except RuntimeError:
+        pytest.skip("no hipcc")
+    for src in build.sources():
+        out = tmp_path / (os.path.basename(src) + ".s")
+        subprocess.run([hipcc, *build.HIPCC_FLAGS, "-I", build.CSRC, "-S", "--cuda-device-only", src, "-o", str(out)],
+                       check=True, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        text = out.read_text()
+        assert not re.search(r"s_set_gpr_idx|v_movrel", text), f"{os.path.basename(src)} uses relative register indexing"
+        spills = [int(m) for m in re.findall(r"\.vgpr_spill_count:\s+(\d+)", text)]
+        assert spills and max(spills) == 0, f"{os.path.basename(src)} spills registers: {spills}"
