@@ -164,12 +164,21 @@ def gated_feed_forward(
     w2: torch.Tensor,
     bias_fused: Optional[torch.Tensor] = None,
     bias2: Optional[torch.Tensor] = None,
+    storage=None,
 ) -> torch.Tensor:
     """fms/modules/feedforward.py:288-297: first half of the fused rows is the gate."""
+    st = _stored(storage)
     hidden = wg1_fused.shape[0] // 2
-    both = linear(x, wg1_fused, bias_fused)
+    both = st(linear(x, wg1_fused, bias_fused))
     gate, up = both[..., :hidden], both[..., hidden:]
-    return linear(silu(gate) * up, w2, bias2)
+    return linear(st(silu(gate) * up), w2, bias2)
+
+
+def _stored(storage):
+    """Rounding to the type in which the reference would hold a tensor (identity for float32)."""
+    if storage is None or storage == torch.float32:
+        return lambda t: t
+    return lambda t: t.to(storage).float()
 
 
 def attention_block(
@@ -181,17 +190,19 @@ def attention_block(
     freqs: torch.Tensor,
     qkv_b: Optional[torch.Tensor] = None,
     dense_b: Optional[torch.Tensor] = None,
+    storage=None,
 ) -> torch.Tensor:
     """fms/modules/attention.py:870-937: project, split [H*D, K*D, K*D], rotate q and k, attend, project."""
+    st = _stored(storage)
     S = x.shape[0]
     H, K, D = cfg.nheads, cfg.kvheads, cfg.head_dim
-    qkv = linear(x, qkv_w, qkv_b)
+    qkv = st(linear(x, qkv_w, qkv_b))
     q, k, v = torch.split(qkv, [H * D, K * D, K * D], dim=-1)
-    q = rope_rotate(q.reshape(S, H, D), positions, freqs)
-    k = rope_rotate(k.reshape(S, K, D), positions, freqs)
+    q = st(rope_rotate(q.reshape(S, H, D), positions, freqs))
+    k = st(rope_rotate(k.reshape(S, K, D), positions, freqs))
     v = v.reshape(S, K, D)
-    mixed = causal_attention(q, k, v)
-    return linear(mixed.reshape(S, H * D), dense_w, dense_b)
+    mixed = st(causal_attention(q, k, v))
+    return st(linear(mixed.reshape(S, H * D), dense_w, dense_b))
 
 
 def forward(
@@ -199,8 +210,16 @@ def forward(
     cfg: PlainConfig,
     ids: List[int],
     first_position: int = 0,
+    storage=None,
 ) -> torch.Tensor:
-    """fms/models/llama.py:137-162, 332-353, 444-445: logits [S, V] of one whole sequence."""
+    """fms/models/llama.py:137-162, 332-353, 444-445: logits [S, V] of one whole sequence.
+
+    storage=torch.bfloat16 rounds every tensor that the reference would hold in its model dtype
+    (the outputs of norms, linears, rotation, attention and the gate product) and computes the
+    rest in float32 as the reference does (norm statistics, rotation).  It serves to size the
+    error that bfloat16 storage alone causes; the residual stream and the logits stay float32.
+    """
+    st = _stored(storage)
     w = {name: t.float() for name, t in weights.items()}
     tokens = torch.as_tensor(ids, dtype=torch.long)
     positions = torch.arange(len(ids)) + first_position
@@ -212,7 +231,7 @@ def forward(
     for i in range(cfg.nlayers):
         p = f"base_model.layers.{i}."
         residual = x
-        h = rms_norm(x, w[p + "ln.weight"], cfg.eps)
+        h = st(rms_norm(x, w[p + "ln.weight"], cfg.eps))
         h = attention_block(
             h,
             positions,
@@ -222,19 +241,21 @@ def forward(
             freqs,
             w.get(p + "attn.in_proj.qkv_fused.bias"),
             w.get(p + "attn.dense.bias"),
+            storage,
         )
         x = h + residual
         residual = x
-        h = rms_norm(x, w[p + "ff_ln.weight"], cfg.eps)
-        h = gated_feed_forward(
+        h = st(rms_norm(x, w[p + "ff_ln.weight"], cfg.eps))
+        h = st(gated_feed_forward(
             h,
             w[p + "ff_sub_layer.wg1_fused.weight"],
             w[p + "ff_sub_layer.w2.weight"],
             w.get(p + "ff_sub_layer.wg1_fused.bias"),
             w.get(p + "ff_sub_layer.w2.bias"),
-        )
+            storage,
+        ))
         x = h + residual
-    x = rms_norm(x, w["base_model.dec_norm.weight"], cfg.eps)
+    x = st(rms_norm(x, w["base_model.dec_norm.weight"], cfg.eps))
     head = w["base_model.embedding.weight"] if cfg.tie_heads and "head.weight" not in w else w["head.weight"]
     return linear(x, head)
 

@@ -218,19 +218,22 @@ def test_long_decoding(lib, folders, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_far_key_decides(lib, folders, dtype, tmp_path):
     """Weights made so that attention is sharp: the logits depend on single far keys, so a key
-    lost at a page border, a split or a slot shows as a large error instead of hiding in an average."""
+    lost at a page border, a split or a slot shows as a large error instead of hiding in an average.
+
+    Sharp attention also amplifies rounding.  For bfloat16 the bound is therefore taken from the
+    plain implementation itself: the error that bfloat16 storage alone causes there."""
     from fms_amd.engine import Engine
+    from fms_amd.weights import write_safetensors
 
     kw = dict(CONFIGS["A"], max_expected_seq_len=1024)
     folder = str(tmp_path / "sharp")
     lib.write_model_folder(folder, lib.LLaMAConfig(**kw), seed=5, std=0.08, norm_std=0.2)
     # scale the query and key projections up: scores spread over tens of units
+    sharpness = 6 if dtype == "float32" else 3
     tensors = P.read_safetensors(os.path.join(folder, "model.safetensors"))
-    from fms_amd.weights import write_safetensors
-
     for k in list(tensors):
         if "q_proj" in k or "k_proj" in k:
-            tensors[k] = (tensors[k].float() * 6).to(torch.bfloat16)
+            tensors[k] = (tensors[k].float() * sharpness).to(torch.bfloat16)
     write_safetensors(os.path.join(folder, "model.safetensors"), [(k, tuple(v.shape), v.dtype) for k, v in tensors.items()],
                       lambda name: tensors[name])
     cfg, weights = P.load_model_folder(folder)
@@ -243,7 +246,15 @@ def test_far_key_decides(lib, folders, dtype, tmp_path):
     for tok in ids[600:]:
         got.append(engine.step([slot], [[tok]], "last"))
     engine.end_sequence(slot)
-    check(torch.cat(got), want, dtype)
+    got = torch.cat(got).float().cpu()
+    if dtype == "float32":
+        check(got, want, dtype)
+    else:
+        storage_error = float((P.forward(weights, cfg, ids, storage=torch.bfloat16) - want).abs().max())
+        scale = float(want.abs().max())
+        assert 0.02 * scale < storage_error < 0.15 * scale  # sharp enough to matter, not so sharp that bfloat16 means nothing
+        err = float((got - want).abs().max())
+        assert err <= 1.5 * storage_error + 0.01 * scale, f"error {err:.3g}; bfloat16 storage alone gives {storage_error:.3g}"
 
 
 # --------------------------------------------------------------------------
