@@ -75,11 +75,11 @@ def main() -> int:
             first = choose(logits, greedy).tolist()
             tokens = first if tokens is None else tokens + first
         for _ in range(warmup):
-            tokens = choose(engine.step(slots, [[t] for t in tokens], "last"), greedy).tolist()
+            tokens = engine.decode_and_choose(slots, tokens, greedy)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(steps):
-            tokens = choose(engine.step(slots, [[t] for t in tokens], "last"), greedy).tolist()
+            tokens = engine.decode_and_choose(slots, tokens, greedy)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         mean_ctx = sum(lens) + batch * (1 + warmup + steps / 2)

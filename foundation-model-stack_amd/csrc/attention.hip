@@ -290,109 +290,172 @@ __global__ void __launch_bounds__(WAVES* WAVE)
 
 // ==========================================================================
 // decode: one query token per sequence.  Grid (split, kv head x head tile,
-// token).  The 16 columns of a wave are query heads that share the kv head.
-// Each block covers `pages_per_block` pages; its waves take them in turn and
-// merge through LDS; blocks of one token merge in attn_decode_merge_kernel.
+// token); a block is ONE wave whose 16 columns are query heads that share the
+// kv head.  A split covers `pages_per_split` pages.  Small blocks in large
+// numbers keep the whole cache of a small batch in flight at once; the loads
+// of a page (keys and values) are issued together before any arithmetic.
+// Splits of one token meet in attn_decode_merge_kernel.
 // ==========================================================================
-#define DECODE_WAVES 4
+template <int MAXDT, int HALVES>
+__device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
+                                            int qlo, int key0, const bf16* __restrict__ kp,
+                                            const bf16* __restrict__ vp, int head_dim, float scale) {
+  // HALVES halves of 32 keys starting at key0 (kp/vp point at the page, `first` is the half inside it)
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int ndt = head_dim / 16;
+  const int nchunk = (head_dim + 31) / 32;
+  const int first = (key0 % PAGE_TOKENS) / 32;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16x4 zero4 = {0, 0, 0, 0};
+  bf16x8 kreg[HALVES][2][(MAXDT + 1) / 2];
+  bf16x4 vreg[HALVES][MAXDT][2];
+#pragma unroll
+  for (int hf = 0; hf < HALVES; ++hf) {
+#pragma unroll
+    for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
+      const int d = c * 32 + g * 8;
+      const bool ok = c < nchunk && d < head_dim;
+      kreg[hf][0][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + r) * head_dim + d) : zero8;
+      kreg[hf][1][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + 16 + r) * head_dim + d) : zero8;
+    }
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt) {
+      const bf16* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + (first + hf) * 32 + g * 4;
+      vreg[hf][dt][0] = dt < ndt ? load_bf16x4(vrow) : zero4;
+      vreg[hf][dt][1] = dt < ndt ? load_bf16x4(vrow + 16) : zero4;
+    }
+  }
+#pragma unroll
+  for (int hf = 0; hf < HALVES; ++hf) {
+    const int k0 = key0 + hf * 32;
+    f32x4 sa = {0.f, 0.f, 0.f, 0.f}, sb = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
+      if (c < nchunk) {
+        sa = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[hf][0][c], qreg[c], sa, 0, 0, 0);
+        sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[hf][1][c], qreg[c], sb, 0, 0, 0);
+      }
+    }
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ja = k0 + g * 4 + i;
+      const int jb = ja + 16;
+      sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] * scale : -INFINITY;
+      sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] * scale : -INFINITY;
+      mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(st.m[0], mx);
+    const float alpha = __expf(st.m[0] - m_new);
+    st.m[0] = m_new;
+    float pa[4], pb[4], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pa[i] = __expf(sa[i] - m_new);
+      pb[i] = __expf(sb[i] - m_new);
+      psum += pa[i] + pb[i];
+    }
+    st.l[0] = st.l[0] * alpha + psum;
+    const bf16x8 pmat = {(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3],
+                         (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt) {
+      if (dt < ndt) {
+        const bf16x4 va = vreg[hf][dt][0], vb = vreg[hf][dt][1];
+        const bf16x8 v = {va[0], va[1], va[2], va[3], vb[0], vb[1], vb[2], vb[3]};
+        st.acc[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat, st.acc[0][dt] * alpha, 0, 0, 0);
+      }
+    }
+  }
+}
 
 template <int MAXDT>
-__global__ void __launch_bounds__(DECODE_WAVES* WAVE)
+__global__ void __launch_bounds__(WAVE)
     attn_decode_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                             float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                            int window, int pages_per_block, int tile_cols) {
-  extern __shared__ float lds[];  // [wave][tile_cols columns][head_dim + 2]
+                            int window, int pages_per_split) {
   const int split = blockIdx.x;
   const int group = nheads / kvheads;
-  const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
+  const int tiles_per_kv = (group + 15) / 16;
   const int kh = blockIdx.y / tiles_per_kv;
   const int ht = blockIdx.y % tiles_per_kv;
   const int t = blockIdx.z;
-  const int wave = threadIdx.x / WAVE;
-  const int lane = threadIdx.x & (WAVE - 1);
+  const int lane = threadIdx.x;
   const int r = lane & 15;
   const int g = lane >> 4;
   const int seq = seq_of_token[t];
-  const int cols = group - ht * tile_cols < tile_cols ? group - ht * tile_cols : tile_cols;  // query heads here
-  const int head0 = kh * group + ht * tile_cols;
+  const int cols = group - ht * 16 < 16 ? group - ht * 16 : 16;  // query heads in this tile
+  const int head0 = kh * group + ht * 16;
   if (seq < 0) {
     if (split == 0)
-      for (int i = threadIdx.x; i < cols * head_dim; i += blockDim.x)
+      for (int i = lane; i < cols * head_dim; i += WAVE)
         out[(size_t)t * out_stride + (size_t)head0 * head_dim + i] = (bf16)0.f;
     return;
   }
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first_split = (lo / PAGE_TOKENS) / pages_per_block;
-  const int last_split = (pos / PAGE_TOKENS) / pages_per_block;
+  const int first_split = (lo / PAGE_TOKENS) / pages_per_split;
+  const int last_split = (pos / PAGE_TOKENS) / pages_per_split;
   if (split < first_split || split > last_split) return;
 
   const int* bt = block_table + (size_t)seq * table_stride;
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
 
-  bf16x8 qreg[1][(MAXDT + 1) / 2];
-  load_query<MAXDT>(qreg[0], r < cols ? q + (size_t)t * q_stride + (size_t)(head0 + r) * head_dim : nullptr, head_dim);
-  const int qpos[1] = {pos};
-  const int qlo[1] = {lo};
+  bf16x8 qreg[(MAXDT + 1) / 2];
+  load_query<MAXDT>(qreg, r < cols ? q + (size_t)t * q_stride + (size_t)(head0 + r) * head_dim : nullptr, head_dim);
 
-  // this block's keys, and the pages of this wave among them
-  int key_lo = split * pages_per_block * PAGE_TOKENS;
-  int key_hi = key_lo + pages_per_block * PAGE_TOKENS - 1;
-  if (key_lo < lo) key_lo = lo;
-  if (key_hi > pos) key_hi = pos;
-  const int block_first_page = key_lo / PAGE_TOKENS;
+  int page_lo = split * pages_per_split;
+  int page_hi = page_lo + pages_per_split - 1;
+  if (page_lo < lo / PAGE_TOKENS) page_lo = lo / PAGE_TOKENS;
+  if (page_hi > pos / PAGE_TOKENS) page_hi = pos / PAGE_TOKENS;
 
   WaveState<MAXDT, 1> st;
   wave_state_init(st);
-  attn_wave_pages<MAXDT, 1>(st, qreg, qpos, qlo, key_lo, key_hi, block_first_page + wave, DECODE_WAVES, bt, k_cache,
-                            v_cache, page_elems, kh, head_dim, scale);
+  for (int pi = page_lo; pi <= page_hi; ++pi) {
+    const size_t phys = (size_t)bt[pi];
+    const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
+    const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
+    if (MAXDT <= 8) {
+      decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale);
+    } else {  // large heads: half a page at a time keeps the loads in registers
+      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale);
+      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, scale);
+    }
+  }
 
-  // ---- merge the waves of the block through LDS -------------------------
   const int ndt = head_dim / 16;
-  const int cstride = head_dim + 2;
   float l = st.l[0];
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
-  if (r < cols) {
-    float* dst = lds + ((size_t)wave * tile_cols + r) * cstride;
-    if (g == 0) {
-      dst[head_dim] = st.m[0];
-      dst[head_dim + 1] = l;
+  if (r >= cols) return;
+  const int head = head0 + r;
+  if (n_splits == 1) {
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    bf16* orow = out + (size_t)t * out_stride + (size_t)head * head_dim;
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt) {
+      if (dt < ndt) {
+        const f32x4 a = st.acc[0][dt];
+        const bf16x4 o = {(bf16)(a[0] * inv), (bf16)(a[1] * inv), (bf16)(a[2] * inv), (bf16)(a[3] * inv)};
+        *reinterpret_cast<bf16x4*>(orow + dt * 16 + g * 4) = o;
+      }
     }
+  } else {
+    const size_t base = ((size_t)t * nheads + head) * n_splits + split;
+    float* prow = part_o + base * head_dim;
 #pragma unroll
     for (int dt = 0; dt < MAXDT; ++dt)
-      if (dt < ndt)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dst[dt * 16 + g * 4 + i] = st.acc[0][dt][i];
-  }
-  __syncthreads();
-  for (int idx = threadIdx.x; idx < cols * head_dim; idx += blockDim.x) {
-    const int c = idx / head_dim;
-    const int d = idx % head_dim;
-    float m = -1e30f;
-#pragma unroll
-    for (int w = 0; w < DECODE_WAVES; ++w) m = fmaxf(m, lds[((size_t)w * tile_cols + c) * cstride + head_dim]);
-    float o = 0.f, lsum = 0.f;
-#pragma unroll
-    for (int w = 0; w < DECODE_WAVES; ++w) {
-      const float* src = lds + ((size_t)w * tile_cols + c) * cstride;
-      const float f = __expf(src[head_dim] - m);
-      o += f * src[d];
-      lsum += f * src[head_dim + 1];
-    }
-    const int head = head0 + c;
-    if (n_splits == 1) {
-      out[(size_t)t * out_stride + (size_t)head * head_dim + d] = (bf16)(lsum > 0.f ? o / lsum : 0.f);
-    } else {
-      const size_t base = ((size_t)t * nheads + head) * n_splits + split;
-      part_o[base * head_dim + d] = o;
-      if (d == 0) {
-        part_ml[base * 2] = m;
-        part_ml[base * 2 + 1] = lsum;
-      }
+      if (dt < ndt) *reinterpret_cast<f32x4*>(prow + dt * 16 + g * 4) = st.acc[0][dt];
+    if (g == 0) {
+      part_ml[base * 2] = st.m[0];
+      part_ml[base * 2 + 1] = l;
     }
   }
 }
@@ -401,14 +464,14 @@ __global__ void __launch_bounds__(DECODE_WAVES* WAVE)
 __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          bf16* __restrict__ out, long out_stride, const int* __restrict__ positions,
                                          const int* __restrict__ seq_of_token, int nheads, int head_dim, int n_splits,
-                                         int window, int pages_per_block) {
+                                         int window, int pages_per_split) {
   const int h = blockIdx.x;
   const int t = blockIdx.y;
   if (seq_of_token[t] < 0) return;  // the decode kernel wrote zeros
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first_split = (lo / PAGE_TOKENS) / pages_per_block;
-  const int last_split = (pos / PAGE_TOKENS) / pages_per_block;
+  const int first_split = (lo / PAGE_TOKENS) / pages_per_split;
+  const int last_split = (pos / PAGE_TOKENS) / pages_per_split;
   const size_t base = ((size_t)t * nheads + h) * n_splits;
   float m = -1e30f;
   for (int s = first_split; s <= last_split; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
@@ -496,31 +559,29 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        long workspace_bytes, const int* positions, const int* seq_of_token,
                                        const int* block_table, int table_stride, const void* k_cache,
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
-                                       float scale, int window, int max_context, int pages_per_block,
+                                       float scale, int window, int max_context, int pages_per_split,
                                        hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
-  FMS_REQUIRE(q_stride % 8 == 0, "attn_decode_bf16: query row stride must keep 16-byte alignment");
-  FMS_REQUIRE(pages_per_block > 0 && max_context > 0, "attn_decode_bf16: bad split sizes");
+  FMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attn_decode_bf16: row strides must keep 16-byte alignment");
+  FMS_REQUIRE(pages_per_split > 0 && max_context > 0, "attn_decode_bf16: bad split sizes");
   FMS_REQUIRE(n_tokens <= 65535, "attn_decode_bf16: %d tokens exceed one launch (65535)", n_tokens);
-  const int n_splits = ceil_div(ceil_div(max_context, PAGE_TOKENS), pages_per_block);
+  const int n_splits = ceil_div(ceil_div(max_context, PAGE_TOKENS), pages_per_split);
   const long need = fmsamd_attn_decode_workspace(n_tokens, nheads, head_dim, n_splits);
   FMS_REQUIRE(workspace_bytes >= need, "attn_decode_bf16: workspace of %ld bytes, %ld needed", workspace_bytes, need);
+  FMS_REQUIRE(need == 0 || ((size_t)workspace % 16) == 0, "attn_decode_bf16: workspace must be 16-byte aligned");
   const int group = nheads / kvheads;
-  const int tile_cols = head_dim > 128 ? 8 : 16;  // keeps the merge buffer within 64 KB of LDS
-  const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
+  const int tiles_per_kv = (group + 15) / 16;
   FMS_REQUIRE((long)kvheads * tiles_per_kv <= 65535, "attn_decode_bf16: too many heads");
   float* part_o = (float*)workspace;
   float* part_ml = part_o ? part_o + (size_t)n_tokens * nheads * n_splits * head_dim : nullptr;
   dim3 grid(n_splits, kvheads * tiles_per_kv, n_tokens);
-  dim3 block(DECODE_WAVES * WAVE);
-  const size_t lds_bytes = (size_t)DECODE_WAVES * tile_cols * (head_dim + 2) * sizeof(float);
 #define FMS_DC(M)                                                                                                    \
-  attn_decode_bf16_kernel<M><<<grid, block, lds_bytes, stream>>>(                                                    \
+  attn_decode_bf16_kernel<M><<<grid, dim3(WAVE), 0, stream>>>(                                                       \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, pages_per_block, tile_cols)
+      window, pages_per_split)
   if (head_dim <= 64)
     FMS_DC(4);
   else if (head_dim <= 128)
@@ -531,9 +592,9 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   FMS_LAUNCH_CHECK("attn_decode_bf16");
   if (n_splits > 1) {
     dim3 mgrid(nheads, n_tokens);
-    attn_decode_merge_kernel<<<mgrid, 64, 0, stream>>>(part_o, part_ml, (bf16*)out, out_stride, positions,
-                                                       seq_of_token, nheads, head_dim, n_splits, window,
-                                                       pages_per_block);
+    attn_decode_merge_kernel<<<mgrid, head_dim <= 64 ? 64 : 128, 0, stream>>>(
+        part_o, part_ml, (bf16*)out, out_stride, positions, seq_of_token, nheads, head_dim, n_splits, window,
+        pages_per_split);
     FMS_LAUNCH_CHECK("attn_decode_merge");
   }
   return 0;

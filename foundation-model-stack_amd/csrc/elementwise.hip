@@ -59,47 +59,92 @@ extern "C" int fmsamd_embed(const int* ids, const void* table, int table_dtype, 
 // With `rows`, output row i is computed from stream row rows[i] and the
 // residual is not written back (the stream is not used again).
 // --------------------------------------------------------------------------
-template <typename BranchT, typename WeightT, typename OutT>
+// VEC consecutive elements as float, from float or bfloat16 storage
+template <int VEC, typename T>
+__device__ __forceinline__ void load_vec(const T* p, float (&v)[VEC]) {
+  if constexpr (VEC == 4 && sizeof(T) == 4) {
+    const f32x4 t = *reinterpret_cast<const f32x4*>(p);
+    v[0] = t[0], v[1] = t[1], v[2] = t[2], v[3] = t[3];
+  } else if constexpr (VEC == 4 && sizeof(T) == 2) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+    v[0] = (float)t[0], v[1] = (float)t[1], v[2] = (float)t[2], v[3] = (float)t[3];
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) v[i] = to_f32(p[i]);
+  }
+}
+
+template <int VEC, typename T>
+__device__ __forceinline__ void store_vec(T* p, const float (&v)[VEC]) {
+  if constexpr (VEC == 4 && sizeof(T) == 4) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{v[0], v[1], v[2], v[3]};
+  } else if constexpr (VEC == 4 && sizeof(T) == 2) {
+    *reinterpret_cast<bf16x4*>(p) = bf16x4{(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+  } else {
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) p[i] = from_f32<T>(v[i]);
+  }
+}
+
+// A thread keeps KEEP vectors of VEC elements in registers (and their weights, fetched before the
+// reduction so that they do not wait for it); a wider row is read again.  The loops over the kept
+// values have compile-time trip counts: the arrays must never be indexed by a run-time value, or
+// they are addressed through relative register indexing.
+template <int VEC, typename BranchT, typename WeightT, typename OutT>
 __global__ void __launch_bounds__(1024) add_norm_kernel(float* __restrict__ resid, const BranchT* __restrict__ branch,
-                                const WeightT* __restrict__ weight, const WeightT* __restrict__ bias,
-                                OutT* __restrict__ out, const int* __restrict__ rows, int width, float eps,
-                                int use_mean) {
+                                                        const WeightT* __restrict__ weight,
+                                                        const WeightT* __restrict__ bias, OutT* __restrict__ out,
+                                                        const int* __restrict__ rows, int width, float eps,
+                                                        int use_mean) {
   __shared__ float scratch[17];
   const int r = rows ? rows[blockIdx.x] : blockIdx.x;
   float* x = resid + (size_t)r * width;
   const BranchT* b = branch ? branch + (size_t)r * width : nullptr;
   OutT* o = out + (size_t)blockIdx.x * width;
 
-  // The first KEEP values of a thread stay in registers; a wider row is read again.  The loops over
-  // the kept values have compile-time trip counts: the array must never be indexed by a run-time
-  // value, or it is addressed through relative register indexing.
-  constexpr int KEEP = 16;
-  float keep[KEEP];
-  const int tail = threadIdx.x + KEEP * blockDim.x;
+  constexpr int KEEP = VEC == 4 ? 4 : 16;
+  const int stride = blockDim.x * VEC;  // elements covered by the block in one sweep
+  float keep[KEEP][VEC], wkeep[KEEP][VEC], bkeep[KEEP][VEC];
+  const int tail = threadIdx.x * VEC + KEEP * stride;
   float sum = 0.f, sq = 0.f;
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * blockDim.x;
-    float v = 0.f;
-    if (i < width) {
-      v = x[i];
+    const int i = threadIdx.x * VEC + n * stride;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) keep[n][e] = 0.f, wkeep[n][e] = 1.f, bkeep[n][e] = 0.f;
+    if (i < width) {  // width is a multiple of VEC
+      load_vec<VEC>(x + i, keep[n]);
+      if (weight) load_vec<VEC>(weight + i, wkeep[n]);
+      if (bias) load_vec<VEC>(bias + i, bkeep[n]);
       if (b) {
-        v += to_f32(b[i]);
-        if (!rows) x[i] = v;
+        float bv[VEC];
+        load_vec<VEC>(b + i, bv);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) keep[n][e] += bv[e];
+        if (!rows) store_vec<VEC>(x + i, keep[n]);
       }
     }
-    keep[n] = v;
-    sum += v;
-    sq += v * v;
-  }
-  for (int i = tail; i < width; i += blockDim.x) {
-    float v = x[i];
-    if (b) {
-      v += to_f32(b[i]);
-      if (!rows) x[i] = v;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      sum += keep[n][e];
+      sq += keep[n][e] * keep[n][e];
     }
-    sum += v;
-    sq += v * v;
+  }
+  for (int i = tail; i < width; i += stride) {
+    float v[VEC];
+    load_vec<VEC>(x + i, v);
+    if (b) {
+      float bv[VEC];
+      load_vec<VEC>(b + i, bv);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[e] += bv[e];
+      if (!rows) store_vec<VEC>(x + i, v);
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      sum += v[e];
+      sq += v[e] * v[e];
+    }
   }
   const bool reread_adds = rows != nullptr && b != nullptr;  // the stream was not updated: add again
   float mean = 0.f;
@@ -108,41 +153,72 @@ __global__ void __launch_bounds__(1024) add_norm_kernel(float* __restrict__ resi
     sq = 0.f;  // second moment about the mean
 #pragma unroll
     for (int n = 0; n < KEEP; ++n) {
-      const int i = threadIdx.x + n * blockDim.x;
-      if (i < width) sq += (keep[n] - mean) * (keep[n] - mean);
+      const int i = threadIdx.x * VEC + n * stride;
+      if (i < width) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) sq += (keep[n][e] - mean) * (keep[n][e] - mean);
+      }
     }
-    for (int i = tail; i < width; i += blockDim.x) {
-      const float v = (reread_adds ? x[i] + to_f32(b[i]) : x[i]) - mean;
-      sq += v * v;
+    for (int i = tail; i < width; i += stride) {
+      float v[VEC];
+      load_vec<VEC>(x + i, v);
+      if (reread_adds) {
+        float bv[VEC];
+        load_vec<VEC>(b + i, bv);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) v[e] += bv[e];
+      }
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) sq += (v[e] - mean) * (v[e] - mean);
     }
   }
   const float ms = block_sum(sq, scratch) / (float)width;
   const float scale = rsqrtf(ms + eps);
 #pragma unroll
   for (int n = 0; n < KEEP; ++n) {
-    const int i = threadIdx.x + n * blockDim.x;
+    const int i = threadIdx.x * VEC + n * stride;
     if (i < width) {
-      float v = (keep[n] - mean) * scale;
-      if (weight) v *= to_f32(weight[i]);
-      if (bias) v += to_f32(bias[i]);
-      o[i] = from_f32<OutT>(v);
+      float v[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[e] = (keep[n][e] - mean) * scale * wkeep[n][e] + bkeep[n][e];
+      store_vec<VEC>(o + i, v);
     }
   }
-  for (int i = tail; i < width; i += blockDim.x) {
-    float v = ((reread_adds ? x[i] + to_f32(b[i]) : x[i]) - mean) * scale;
-    if (weight) v *= to_f32(weight[i]);
-    if (bias) v += to_f32(bias[i]);
-    o[i] = from_f32<OutT>(v);
+  for (int i = tail; i < width; i += stride) {
+    float v[VEC], wv[VEC], bv[VEC];
+    load_vec<VEC>(x + i, v);
+    if (reread_adds) {
+      load_vec<VEC>(b + i, bv);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) v[e] += bv[e];
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) wv[e] = 1.f, bv[e] = 0.f;
+    if (weight) load_vec<VEC>(weight + i, wv);
+    if (bias) load_vec<VEC>(bias + i, bv);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) v[e] = (v[e] - mean) * scale * wv[e] + bv[e];
+    store_vec<VEC>(o + i, v);
   }
 }
 
 template <typename BranchT, typename WeightT, typename OutT>
 static void launch_add_norm(float* resid, const void* branch, const void* weight, const void* bias, void* out,
                             const int* rows, int n_out, int width, float eps, int use_mean, hipStream_t stream) {
-  const int threads = width > 4096 ? 1024 : (width >= 2048 ? 256 : (width >= 512 ? 128 : 64));
-  add_norm_kernel<BranchT, WeightT, OutT><<<n_out, threads, 0, stream>>>(
-      resid, (const BranchT*)branch, (const WeightT*)weight, (const WeightT*)bias, (OutT*)out, rows, width, eps,
-      use_mean);
+  const bool aligned = (((size_t)resid | (size_t)branch | (size_t)weight | (size_t)bias | (size_t)out) & 15) == 0;
+  if (width % 4 == 0 && aligned) {
+    // 4 vectors of 4 per thread cover the row up to 16 elements per thread; wider rows take more threads
+    int threads = (width / 16 + 63) / 64 * 64;
+    threads = threads < 64 ? 64 : (threads > 1024 ? 1024 : threads);
+    add_norm_kernel<4, BranchT, WeightT, OutT><<<n_out, threads, 0, stream>>>(
+        resid, (const BranchT*)branch, (const WeightT*)weight, (const WeightT*)bias, (OutT*)out, rows, width, eps,
+        use_mean);
+  } else {
+    const int threads = width > 4096 ? 1024 : (width >= 2048 ? 256 : (width >= 512 ? 128 : 64));
+    add_norm_kernel<1, BranchT, WeightT, OutT><<<n_out, threads, 0, stream>>>(
+        resid, (const BranchT*)branch, (const WeightT*)weight, (const WeightT*)bias, (OutT*)out, rows, width, eps,
+        use_mean);
+  }
 }
 
 extern "C" int fmsamd_add_norm(float* resid, const void* branch, int act_dtype, const void* weight, const void* bias,
@@ -266,5 +342,22 @@ extern "C" int fmsamd_bias_add(void* x, int dtype, const void* bias, int bias_dt
   else
     FMS_REQUIRE(false, "bias_add: unknown dtypes");
   FMS_LAUNCH_CHECK("bias_add");
+  return 0;
+}
+
+// --------------------------------------------------------------------------
+// positions[i] += 1 for the live rows of a fixed-size decode batch, so that a
+// captured step can be replayed without the host touching its index data
+// --------------------------------------------------------------------------
+__global__ void advance_positions_kernel(int* __restrict__ positions, const int* __restrict__ seq_of_token, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n && seq_of_token[i] >= 0) positions[i] += 1;
+}
+
+extern "C" int fmsamd_advance_positions(int* positions, const int* seq_of_token, int n, hipStream_t stream) {
+  if (n == 0) return 0;
+  FMS_REQUIRE(n > 0, "advance_positions: negative count");
+  advance_positions_kernel<<<ceil_div(n, 256), 256, 0, stream>>>(positions, seq_of_token, n);
+  FMS_LAUNCH_CHECK("advance_positions");
   return 0;
 }

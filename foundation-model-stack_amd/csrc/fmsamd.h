@@ -39,6 +39,9 @@ int fmsamd_add_norm(float* resid, const void* branch, int act_dtype, const void*
 int fmsamd_gated_act(const void* gu, const void* bias, int bias_dtype, void* out, int dtype, int n_tokens, int hidden,
                      int act, hipStream_t stream);
 
+// positions[i] += 1 where seq_of_token[i] >= 0
+int fmsamd_advance_positions(int* positions, const int* seq_of_token, int n, hipStream_t stream);
+
 int fmsamd_cast(const void* in, int in_dtype, void* out, int out_dtype, long n, hipStream_t stream);
 int fmsamd_bias_add(void* x, int dtype, const void* bias, int bias_dtype, int rows, int cols, hipStream_t stream);
 
@@ -66,13 +69,13 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                              hipStream_t stream);
 
-// bfloat16 decode: one token per sequence, keys split over blocks of `pages_per_block` pages
+// bfloat16 decode: one token per sequence, keys split over one-wave blocks of `pages_per_split` pages
 long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits);
 int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_stride, void* workspace,
                             long workspace_bytes, const int* positions, const int* seq_of_token,
                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
-                            int max_context, int pages_per_block, hipStream_t stream);
+                            int max_context, int pages_per_split, hipStream_t stream);
 
 // c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
 int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,
@@ -84,9 +87,18 @@ int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* 
 int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                   int out_dtype, long ldo, int M, int hidden, int K, int act, hipStream_t stream);
 
+// tuning aid: the skinny product (M <= 16, bfloat16 out) with explicit launch shape
+int fmsamd_gemm_skinny_variant(const void* x, long ldx, const void* w, void* out, long ldo, int M, int N, int K,
+                               int waves, int unr, int ntb, hipStream_t stream);
+
 // token choice; rng_state is [rows][2] uint64 (seed, counter), advanced by the kernel
 int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature, int top_k,
                   void* rng_state, int* out_tokens, hipStream_t stream);
+
+// greedy choice over many blocks per row; workspace of fmsamd_argmax_workspace(rows, vocab) bytes
+long fmsamd_argmax_workspace(int rows, int vocab);
+int fmsamd_argmax(const float* logits, long ld, int rows, int vocab, void* workspace, long workspace_bytes,
+                  int* out_tokens, hipStream_t stream);
 
 #ifdef __cplusplus
 }

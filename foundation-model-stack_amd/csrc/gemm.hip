@@ -202,7 +202,9 @@ __device__ __forceinline__ float sk_activate(float x, int kind) {
 // MT : 16-row tiles of x.
 // GATED: the second tile is the "up" half; out = act(first) * second, N is the hidden size.
 // SK_WAVES: waves of a block (8, or 4 when NTB*MT > 4 so that the LDS buffer stays under 64 KB).
-template <int SK_WAVES, int NTB, int MT, bool GATED, typename OutT, typename BiasT>
+// UNR: chunks of 64 k-values whose loads a wave issues before it multiplies: what keeps enough
+// bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 2 loads of 16 bytes outstanding).
+template <int SK_WAVES, int UNR, int NTB, int MT, bool GATED, typename OutT, typename BiasT>
 __global__ void __launch_bounds__(SK_WAVES* WAVE)
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act) {
@@ -235,29 +237,35 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 #pragma unroll
     for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // K in chunks of 64: lane group g covers k = chunk*64 + g*16 .. +16 (two MFMA steps)
+  // K in chunks of 64: lane group g covers k = chunk*64 + g*16 .. +16 (two MFMA steps).
+  // A wave takes UNR neighbouring chunks at a time.
   const int nchunks = (K + 63) / 64;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int ch = wave; ch < nchunks; ch += SK_WAVES) {
-    const int k = ch * 64 + g * 16;
-    bf16x8 wa[NTB], wb[NTB], xa[MT], xb[MT];
+  for (int ch0 = wave * UNR; ch0 < nchunks; ch0 += SK_WAVES * UNR) {
+    bf16x8 wa[UNR][NTB], wb[UNR][NTB], xa[UNR][MT], xb[UNR][MT];
 #pragma unroll
-    for (int t = 0; t < NTB; ++t) {
-      wa[t] = (wok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k) : zero;
-      wb[t] = (wok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k + 8) : zero;
-    }
+    for (int u = 0; u < UNR; ++u) {
+      const int k = (ch0 + u) * 64 + g * 16;
 #pragma unroll
-    for (int t = 0; t < MT; ++t) {
-      xa[t] = (xok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k) : zero;
-      xb[t] = (xok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k + 8) : zero;
-    }
-#pragma unroll
-    for (int i = 0; i < NTB; ++i)
-#pragma unroll
-      for (int j = 0; j < MT; ++j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[i], xa[j], acc[i][j], 0, 0, 0);
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[i], xb[j], acc[i][j], 0, 0, 0);
+      for (int t = 0; t < NTB; ++t) {
+        wa[u][t] = (wok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k) : zero;
+        wb[u][t] = (wok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k + 8) : zero;
       }
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        xa[u][t] = (xok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k) : zero;
+        xb[u][t] = (xok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k + 8) : zero;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < UNR; ++u)
+#pragma unroll
+      for (int i = 0; i < NTB; ++i)
+#pragma unroll
+        for (int j = 0; j < MT; ++j) {
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][i], xa[u][j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[u][i], xb[u][j], acc[i][j], 0, 0, 0);
+        }
   }
 
   // partial tiles meet in LDS: red[wave][tile n][tile m][n row][m column]
@@ -303,8 +311,9 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
                           hipStream_t stream) {
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
   constexpr int SK_WAVES = NTB * MT > 4 ? 4 : 8;
-#define FMS_SK(O, B)                                                                             \
-  skinny_bf16_kernel<SK_WAVES, NTB, MT, GATED, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(    \
+  constexpr int UNR = (NTB + MT) <= 2 ? 4 : ((NTB + MT) <= 4 ? 2 : 1);
+#define FMS_SK(O, B)                                                                                  \
+  skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, GATED, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(    \
       (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act)
   if (out_dtype == FMS_BF16) {
     if (fb)
@@ -364,4 +373,26 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
 #undef FMS_LG
   FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
   return 0;
+}
+
+// Tuning aid: the plain skinny product (M <= 16, bfloat16 out, no bias) with an explicit choice of
+// waves per block, chunks in flight per wave and tiles per block.
+template <int W, int U, int NTB>
+static void launch_variant(const void* x, long ldx, const void* w, void* out, long ldo, int M, int N, int K,
+                           hipStream_t stream) {
+  const int blocks = ceil_div(N, 16 * NTB);
+  skinny_bf16_kernel<W, U, NTB, 1, false, bf16, bf16><<<blocks, W * WAVE, 0, stream>>>(
+      (const bf16*)x, ldx, (const bf16*)w, (const bf16*)nullptr, (bf16*)out, ldo, M, N, K, 0, 0);
+}
+
+extern "C" int fmsamd_gemm_skinny_variant(const void* x, long ldx, const void* w, void* out, long ldo, int M, int N,
+                                          int K, int waves, int unr, int ntb, hipStream_t stream) {
+  FMS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_variant: bad sizes");
+#define FMS_V(W, U, T) \
+  if (waves == W && unr == U && ntb == T) { launch_variant<W, U, T>(x, ldx, w, out, ldo, M, N, K, stream); FMS_LAUNCH_CHECK("gemm_skinny_variant"); return 0; }
+  FMS_V(4, 1, 1) FMS_V(4, 2, 1) FMS_V(4, 4, 1) FMS_V(4, 8, 1) FMS_V(8, 1, 1) FMS_V(8, 2, 1) FMS_V(8, 4, 1) FMS_V(8, 8, 1)
+  FMS_V(16, 1, 1) FMS_V(16, 2, 1) FMS_V(16, 4, 1) FMS_V(16, 8, 1)
+  FMS_V(4, 1, 2) FMS_V(4, 2, 2) FMS_V(4, 4, 2) FMS_V(8, 1, 2) FMS_V(8, 2, 2) FMS_V(8, 4, 2) FMS_V(16, 1, 2) FMS_V(16, 2, 2) FMS_V(16, 4, 2)
+#undef FMS_V
+  FMS_REQUIRE(false, "gemm_skinny_variant: no variant waves=%d unr=%d ntb=%d", waves, unr, ntb);
 }

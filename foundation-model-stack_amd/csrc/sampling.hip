@@ -149,6 +149,79 @@ __global__ void __launch_bounds__(SMP_THREADS)
   if (sh_arg < 0 && tid == 0) out_tokens[row] = 0;
 }
 
+// ---- greedy over a large vocabulary: many blocks per row, then one -------------------------
+#define ARG_THREADS 256
+#define ARG_CHUNK 2048  // logits per block of the first stage
+
+__global__ void __launch_bounds__(ARG_THREADS)
+    argmax_partial_kernel(const float* __restrict__ logits, long ld, int vocab, float* __restrict__ part_val,
+                          int* __restrict__ part_idx, int chunks) {
+  __shared__ float scratch[17];
+  __shared__ int sh_arg;
+  const int row = blockIdx.y, chunk = blockIdx.x;
+  const float* x = logits + (size_t)row * ld;
+  const int begin = chunk * ARG_CHUNK;
+  const int end = begin + ARG_CHUNK < vocab ? begin + ARG_CHUNK : vocab;
+  float best = -INFINITY;
+  int arg = 0x7fffffff;
+  for (int i = begin + threadIdx.x; i < end; i += ARG_THREADS) {
+    const float v = x[i];
+    if (v > best || (v == best && i < arg)) best = v, arg = i;
+  }
+  const float mx = block_max(best, scratch);
+  if (threadIdx.x == 0) sh_arg = 0x7fffffff;
+  __syncthreads();
+  if (best == mx && arg != 0x7fffffff) atomicMin(&sh_arg, arg);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    part_val[(size_t)row * chunks + chunk] = mx;
+    part_idx[(size_t)row * chunks + chunk] = sh_arg;
+  }
+}
+
+__global__ void __launch_bounds__(ARG_THREADS)
+    argmax_final_kernel(const float* __restrict__ part_val, const int* __restrict__ part_idx, int chunks,
+                        int* __restrict__ out_tokens) {
+  __shared__ float scratch[17];
+  __shared__ int sh_arg;
+  const int row = blockIdx.x;
+  float best = -INFINITY;
+  int arg = 0x7fffffff;
+  for (int c = threadIdx.x; c < chunks; c += ARG_THREADS) {
+    const float v = part_val[(size_t)row * chunks + c];
+    const int i = part_idx[(size_t)row * chunks + c];
+    if (v > best || (v == best && i < arg)) best = v, arg = i;
+  }
+  const float mx = block_max(best, scratch);
+  if (threadIdx.x == 0) sh_arg = 0x7fffffff;
+  __syncthreads();
+  if (best == mx && arg != 0x7fffffff) atomicMin(&sh_arg, arg);
+  __syncthreads();
+  if (threadIdx.x == 0) out_tokens[row] = sh_arg == 0x7fffffff ? 0 : sh_arg;
+}
+
+extern "C" long fmsamd_argmax_workspace(int rows, int vocab) {
+  return (long)rows * ceil_div(vocab, ARG_CHUNK) * 8;
+}
+
+// greedy choice with a workspace of fmsamd_argmax_workspace(rows, vocab) bytes
+extern "C" int fmsamd_argmax(const float* logits, long ld, int rows, int vocab, void* workspace, long workspace_bytes,
+                             int* out_tokens, hipStream_t stream) {
+  if (rows == 0) return 0;
+  FMS_REQUIRE(rows > 0 && vocab > 0 && ld >= vocab, "argmax: bad sizes rows=%d vocab=%d ld=%ld", rows, vocab, ld);
+  FMS_REQUIRE(rows <= 65535, "argmax: %d rows exceed one launch", rows);
+  const int chunks = ceil_div(vocab, ARG_CHUNK);
+  FMS_REQUIRE(workspace != nullptr && workspace_bytes >= fmsamd_argmax_workspace(rows, vocab),
+              "argmax: workspace of %ld bytes, %ld needed", workspace_bytes, fmsamd_argmax_workspace(rows, vocab));
+  float* part_val = (float*)workspace;
+  int* part_idx = (int*)(part_val + (size_t)rows * chunks);
+  argmax_partial_kernel<<<dim3(chunks, rows), ARG_THREADS, 0, stream>>>(logits, ld, vocab, part_val, part_idx, chunks);
+  FMS_LAUNCH_CHECK("argmax_partial");
+  argmax_final_kernel<<<rows, ARG_THREADS, 0, stream>>>(part_val, part_idx, chunks, out_tokens);
+  FMS_LAUNCH_CHECK("argmax_final");
+  return 0;
+}
+
 extern "C" int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature,
                              int top_k, void* rng_state, int* out_tokens, hipStream_t stream) {
   if (rows == 0) return 0;

@@ -1,0 +1,121 @@
+"""Decode steps as a captured HIP graph.
+
+One decode step of a batch is some hundred small launches; replaying them as a
+graph takes the launch cost and the host's work out of the step.  A graph is
+captured for a fixed number of rows (the batch padded up to a bucket; padding
+rows carry sequence -1 and are skipped by the kernels) and a fixed upper bound
+of the context length (it sizes the split of the attention kernel).  Its index
+data lives in static device buffers: the sampled tokens are written where the
+next step reads its input, positions advance on the device, and the host only
+writes a block-table row when a sequence gets a new page.
+
+No memset is recorded into a graph (fill kernels only), and a graph is only
+used when every part of the model says it can be captured.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache import PAGE_TOKENS, pages_for
+from ..kernels import ops
+from .batch import StepBatch
+
+ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
+CONTEXT_BUCKET = 1024
+
+
+def row_bucket(n: int) -> int:
+    for b in ROW_BUCKETS:
+        if n <= b:
+            return b
+    return -(-n // 64) * 64
+
+
+def context_bucket(n: int, limit: int) -> int:
+    return min(-(-n // CONTEXT_BUCKET) * CONTEXT_BUCKET, max(limit, 1))
+
+
+class DecodeGraph:
+    def __init__(self, engine, rows: int, max_context: int, sampling):
+        self.engine, self.rows, self.max_context, self.sampling = engine, rows, max_context, sampling
+        dev = engine.device
+        cache = engine.cache
+        self.table_width = pages_for(cache.max_seq_len)
+        self.tokens = torch.zeros(rows, dtype=torch.int32, device=dev)
+        self.positions = torch.zeros(rows, dtype=torch.int32, device=dev)
+        self.seq_of_token = torch.full((rows,), -1, dtype=torch.int32, device=dev)
+        self.slot_ids = torch.zeros(rows, dtype=torch.int32, device=dev)
+        self.seq_starts = torch.arange(rows + 1, dtype=torch.int32, device=dev)
+        self.logit_rows = torch.arange(rows, dtype=torch.int32, device=dev)
+        self.tables = {g: torch.zeros(rows, self.table_width, dtype=torch.int32, device=dev) for g in range(len(cache.groups))}
+        self.rng = torch.zeros(rows, 2, dtype=torch.int64, device=dev)
+        self.batch = StepBatch(
+            n_tokens=rows, n_seqs=rows, slots=[], q_lens=[1] * rows, starts=[0] * rows, is_decode=True,
+            max_context=max_context, token_ids=self.tokens, positions=self.positions, seq_of_token=self.seq_of_token,
+            slot_ids=self.slot_ids, seq_starts=self.seq_starts, block_tables=self.tables, qblock_start=None,
+            qblock_len=None, logit_rows=self.logit_rows, n_logit_rows=rows,
+        )
+        # what the static buffers currently describe
+        self.slots: Tuple[int, ...] = ()
+        self.next_tokens: Optional[List[int]] = None  # tokens now in self.tokens (the last step's choices)
+        self.n_pages: List[int] = []
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+
+    def _run(self) -> None:
+        logits = self.engine.model.forward(self.batch, self.engine.cache)
+        s = self.sampling
+        ops.sample(logits, s.do_sample, s.temperature, s.top_k or 0, self.rng if s.do_sample else None, out=self.tokens)
+        ops.advance_positions_(self.positions, self.seq_of_token)
+
+    def capture(self) -> None:
+        # Padding rows only (sequence -1): nothing is written to the cache while warming up and capturing.
+        self.seq_of_token.fill_(-1)
+        self.slots, self.next_tokens = (), None
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            self._run()  # warm-up: lazy initialisation and allocator growth happen outside the capture
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self._run()
+        torch.cuda.synchronize()
+
+    def load(self, slots: Sequence[int], tokens: Sequence[int], positions: Sequence[int], seeds, counters) -> None:
+        """Describe a new batch composition in the static buffers (one small copy each)."""
+        n = len(slots)
+        cache = self.engine.cache
+        pad = self.rows - n
+        dev = self.engine.device
+        self.tokens.copy_(torch.tensor(list(tokens) + [0] * pad, dtype=torch.int32), non_blocking=True)
+        self.positions.copy_(torch.tensor(list(positions) + [0] * pad, dtype=torch.int32), non_blocking=True)
+        self.seq_of_token.copy_(torch.tensor(list(range(n)) + [-1] * pad, dtype=torch.int32), non_blocking=True)
+        self.slot_ids.copy_(torch.tensor(list(slots) + [0] * pad, dtype=torch.int32), non_blocking=True)
+        for g, table in self.tables.items():
+            host = cache.block_table(g, slots, n_columns=self.table_width)
+            table[:n].copy_(host, non_blocking=True)
+        if self.sampling.do_sample:
+            rng = [[int(s), int(c)] for s, c in zip(seeds, counters)] + [[0, 0]] * pad
+            self.rng.copy_(torch.tensor(rng, dtype=torch.int64), non_blocking=True)
+        self.slots = tuple(slots)
+        self.n_pages = [pages_for(cache.length(s)) for s in slots]
+
+    def refresh_pages(self) -> None:
+        """Write the block-table rows of sequences that got a new page since the last step."""
+        cache = self.engine.cache
+        for row, slot in enumerate(self.slots):
+            n = pages_for(cache.length(slot))
+            if n != self.n_pages[row]:
+                for g, table in self.tables.items():
+                    table[row].copy_(cache.block_table(g, [slot], n_columns=self.table_width)[0], non_blocking=True)
+                self.n_pages[row] = n
+
+    def replay(self) -> List[int]:
+        self.graph.replay()
+        out = self.tokens[: len(self.slots)].tolist()
+        self.next_tokens = out
+        return out

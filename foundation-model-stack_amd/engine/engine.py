@@ -9,20 +9,27 @@ no padding: tokens of all sequences are laid end to end.
 
 from __future__ import annotations
 
-from typing import List, Optional, Sequence, Union
+from typing import List, Optional, Sequence, Union  # noqa: F401
 
 import torch
 
+import os
+
 from ..cache import CacheFull, pages_for
 from ..kernels import ops
+from ..sampling import SamplingParams, choose
 from .batch import StepBatch, build_batch
+from .decode_graph import DecodeGraph, context_bucket, row_bucket
 from .model import DecoderModel
 
 
 class Engine:
-    def __init__(self, model: DecoderModel, max_tokens: Optional[int] = None, max_slots: Optional[int] = None):
+    def __init__(self, model: DecoderModel, max_tokens: Optional[int] = None, max_slots: Optional[int] = None,
+                 use_graphs: Optional[bool] = None):
         """max_tokens: the most tokens live sequences hold at a time, each rounded up to a page of 64
-        (default: one sequence of the model's full length).  max_slots: the most live sequences."""
+        (default: one sequence of the model's full length).  max_slots: the most live sequences.
+        use_graphs: replay decode steps as captured HIP graphs (default: yes, if every part allows it
+        and the environment variable FMS_AMD_NO_GRAPHS is not set)."""
         if model.device is None:
             raise RuntimeError("the model has no weights on a device yet (use get_model)")
         self.model = model
@@ -34,6 +41,10 @@ class Engine:
         self.cache = model.make_cache(max_tokens, max_slots)
         self.qblock = ops.prefill_qblock()
         self.vocab = model.spec.vocab
+        if use_graphs is None:
+            use_graphs = not os.environ.get("FMS_AMD_NO_GRAPHS")
+        self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", True) for p in model.walk())
+        self._graphs = {}
 
     # ---- sequences ---------------------------------------------------------
     def new_sequence(self) -> int:
@@ -61,6 +72,50 @@ class Engine:
         if batch.n_tokens == 0:
             return torch.empty(0, self.vocab, dtype=torch.float32, device=self.device)
         return self.model.forward(batch, self.cache)
+
+    def decode_and_choose(
+        self,
+        slots: Sequence[int],
+        tokens: Sequence[int],
+        sampling: SamplingParams,
+        seeds: Optional[Sequence[int]] = None,
+        counters: Optional[Sequence[int]] = None,
+    ) -> List[int]:
+        """One decode step and the choice of the next token for every sequence: `tokens[b]` is appended to
+        `slots[b]`, the chosen tokens come back as host integers.  Replays a captured graph when it can."""
+        slots = [int(s) for s in slots]
+        tokens = [int(t) for t in tokens]
+        if not self.use_graphs:
+            logits = self.step(slots, [[t] for t in tokens], "last")
+            return choose(logits, sampling, seeds, counters).tolist()
+        if len(set(slots)) != len(slots) or len(tokens) != len(slots):
+            raise ValueError("one token per sequence, each sequence once")
+        for t in tokens:
+            if not 0 <= t < self.vocab:
+                raise IndexError(f"token id {t} is outside the vocabulary of {self.vocab}")
+        for group in self.cache.groups:
+            if group.need.window == 0:
+                need = sum(1 for s in slots if self.cache.length(s) % 64 == 0)
+                if need > group.pool.n_free:
+                    raise CacheFull(f"the step needs {need} more cache pages, {group.pool.n_free} are free")
+        for s in slots:
+            if self.cache.length(s) + 1 > self.cache.max_seq_len:
+                raise IndexError(f"sequence in slot {s} has reached the model's {self.cache.max_seq_len} positions")
+        positions = [self.cache.extend(s, 1) for s in slots]
+        rows = row_bucket(len(slots))
+        ctx = context_bucket(max(positions) + 1, self.cache.max_seq_len)
+        key = (rows, ctx, sampling.do_sample, float(sampling.temperature), int(sampling.top_k or 0))
+        graph = self._graphs.get(key)
+        if graph is None:
+            for old in [k for k in self._graphs if k[0] == rows and k[2:] == key[2:]]:
+                del self._graphs[old]  # a longer context replaces the graph of the shorter one
+            graph = self._graphs[key] = DecodeGraph(self, rows, ctx, sampling)
+            graph.capture()
+        if graph.slots == tuple(slots) and graph.next_tokens == tokens:
+            graph.refresh_pages()
+        else:
+            graph.load(slots, tokens, positions, seeds or [0] * len(slots), counters or [0] * len(slots))
+        return graph.replay()
 
     def prepare(self, slots, tokens, want) -> StepBatch:
         slots = [int(s) for s in slots]

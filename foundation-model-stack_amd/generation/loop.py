@@ -87,6 +87,7 @@ def generate_requests(
         seeds = [request_seed(seed, r) for r in request_ids]
         return choose(logits, sampling, seeds, counters).tolist()
 
+    fused = chooser is None and hasattr(engine, "decode_and_choose")
     for batch in plan_batches([len(p) for p in prompts], max_new_tokens, cache.max_tokens, max_batch, cache.max_seq_len):
         slots = {r: engine.new_sequence() for r in batch}
         alive = list(batch)
@@ -95,8 +96,14 @@ def generate_requests(
         try:
             while alive:
                 t0 = time.time()
-                logits = engine.step([slots[r] for r in alive], [feed[r] for r in alive], "last")
-                tokens = pick(logits, alive, [len(results[r]) for r in alive])
+                if fused and step_no > 0:
+                    # decode: the step and the choice in one call (a captured graph when the engine has one)
+                    tokens = engine.decode_and_choose(
+                        [slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
+                        [request_seed(seed, r) for r in alive], [len(results[r]) for r in alive])
+                else:
+                    logits = engine.step([slots[r] for r in alive], [feed[r] for r in alive], "last")
+                    tokens = pick(logits, alive, [len(results[r]) for r in alive])
                 if step_times is not None:
                     step_times.append(time.time() - t0)
                 if on_step is not None:

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "fmsamd_add_norm": [P, P, I, P, P, I, P, P, I, I, F, I, P],
     "fmsamd_gated_act": [P, P, I, P, I, I, I, I, P],
     "fmsamd_cast": [P, I, P, I, L, P],
+    "fmsamd_advance_positions": [P, P, I, P],
     "fmsamd_bias_add": [P, I, P, I, I, I, P],
     "fmsamd_rope_table": [P, P, P, I, I, P],
     "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, P],
@@ -39,7 +40,9 @@ _SIGNATURES = {
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
     "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
     "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P],
+    "fmsamd_gemm_skinny_variant": [P, L, P, P, L, I, I, I, I, I, I, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
+    "fmsamd_argmax": [P, L, I, I, P, L, P, P],
 }
 
 
@@ -77,6 +80,8 @@ def load(verbose: bool = True) -> ctypes.CDLL:
             fn.restype = c_int
         lib.fmsamd_attn_prefill_qblock.restype = c_int
         lib.fmsamd_attn_prefill_qblock.argtypes = []
+        lib.fmsamd_argmax_workspace.restype = c_long
+        lib.fmsamd_argmax_workspace.argtypes = [I, I]
         lib.fmsamd_attn_decode_workspace.restype = c_long
         lib.fmsamd_attn_decode_workspace.argtypes = [I, I, I, I]
         lib.path = path

@@ -132,6 +132,16 @@ def cast(x: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def advance_positions_(positions: torch.Tensor, seq_of_token: torch.Tensor) -> None:
+    """positions += 1 on the live rows (seq_of_token >= 0) of a fixed-size decode batch."""
+    _need_cuda(positions, seq_of_token)
+    _need_i32("positions", positions)
+    _need_i32("seq_of_token", seq_of_token)
+    if positions.numel() != seq_of_token.numel():
+        raise ValueError("positions and seq_of_token must have one entry per row")
+    check(load().fmsamd_advance_positions(positions.data_ptr(), seq_of_token.data_ptr(), positions.numel(), _stream()))
+
+
 def bias_add_(x: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     _need_cuda(x, bias)
     if x.dim() != 2 or not x.is_contiguous() or bias.shape != (x.shape[1],) or not bias.is_contiguous():
@@ -281,12 +291,12 @@ def attention(
 
 
 def decode_pages_per_block(rows: int, n_pages: int) -> int:
-    """How many pages one block of the decode kernel takes: few when there are few (token, kv head)
-    pairs, so that the keys of a long context are spread over many blocks; at most 4 per wave."""
-    target_blocks = 1024
-    splits_wanted = max(1, target_blocks // max(rows, 1))
-    per_block = max(1, -(-n_pages // splits_wanted))
-    return min(max(per_block, 4), 16) if n_pages > 4 else max(1, min(per_block, 4))
+    """How many pages one wave of the decode kernel takes: one, unless that would make more than
+    some ten thousand waves or more than 64 partial results per token to merge."""
+    per_split = 1
+    while rows * -(-n_pages // per_split) > 16384 or -(-n_pages // per_split) > 64:
+        per_split *= 2
+    return per_split
 
 
 def prefill_qblock() -> int:
@@ -297,8 +307,8 @@ def prefill_qblock() -> int:
 # matrix products
 # --------------------------------------------------------------------------
 SKINNY_MAX_ROWS = 64
-# Above this many rows the bfloat16 product goes to the vendor library (hipBLASLt through torch.matmul).
-LIBRARY_GEMM_MIN_ROWS = 65
+# Up to this many rows the skinny kernel streams weights faster than the vendor library does.
+SKINNY_FAST_ROWS = 32
 
 
 def linear(
@@ -310,9 +320,10 @@ def linear(
 ) -> torch.Tensor:
     """x [M, K] @ weight[N, K]^T (+ bias) -> [M, N].
 
-    float32 x float32: the FMA kernel (true 32-bit).  bfloat16 x bfloat16: the skinny kernel up
-    to 64 rows; above that the vendor library for bfloat16 output (as the reference's nn.Linear
-    does), or this package's MFMA kernel when float32 output is wanted or allow_library is False.
+    float32 x float32: the FMA kernel (true 32-bit).  bfloat16 x bfloat16: the weight-streaming
+    skinny kernel up to 32 rows; above that the vendor library (hipBLASLt through torch.matmul,
+    as the reference's nn.Linear does) for bfloat16 output, or this package's MFMA kernels when
+    float32 output is wanted or allow_library is False.
     A float32 weight with bfloat16 activations (a tensor the checkpoint keeps in 32-bit) runs the
     float32 kernel on up-cast activations.
     """
@@ -344,12 +355,12 @@ def linear(
     if K % 8 or x.stride(0) % 8:
         raise ValueError(f"bfloat16 products need K (={K}) and the row stride (={x.stride(0)}) to be multiples of 8")
     bcode = _code(bias.dtype) if bias is not None else 0
-    if M <= SKINNY_MAX_ROWS:
+    if M <= SKINNY_FAST_ROWS or (M <= SKINNY_MAX_ROWS and not (allow_library and out_dtype == torch.bfloat16)):
         out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         check(lib.fmsamd_gemm_skinny_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), bcode, out.data_ptr(),
                                           _code(out_dtype), out.stride(0), M, N, K, _stream()))
         return out
-    if allow_library and out_dtype == torch.bfloat16 and M >= LIBRARY_GEMM_MIN_ROWS:
+    if allow_library and out_dtype == torch.bfloat16:
         out = torch.matmul(x, weight.t())  # vendor library GEMM, float32 accumulation
         if bias is not None:
             bias_add_(out, bias)
@@ -368,7 +379,7 @@ def gated_linear(
     if weight.shape[0] % 2:
         raise ValueError("the stacked gate/up weight needs an even number of rows")
     hidden = weight.shape[0] // 2
-    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M <= SKINNY_MAX_ROWS:
+    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M <= (SKINNY_FAST_ROWS if allow_library else SKINNY_MAX_ROWS):
         _need_cuda(x, weight, bias)
         _rows2d("x", x)
         K = x.shape[1]
@@ -411,6 +422,12 @@ def sample(
         out = torch.empty(rows, dtype=torch.int32, device=logits.device)
     elif out.dtype != torch.int32 or out.numel() < rows or not out.is_contiguous():
         raise ValueError("out must be a contiguous int32 tensor with an entry per row")
+    if not do_sample and vocab > 4096:
+        lib = load()
+        nbytes = lib.fmsamd_argmax_workspace(rows, vocab)
+        ws = torch.empty(nbytes // 4, dtype=torch.float32, device=logits.device)
+        check(lib.fmsamd_argmax(logits.data_ptr(), logits.stride(0), rows, vocab, ws.data_ptr(), nbytes, out.data_ptr(), _stream()))
+        return out
     check(load().fmsamd_sample(logits.data_ptr(), logits.stride(0), rows, vocab, int(bool(do_sample)), float(temperature),
                                int(top_k or 0), _ptr(rng_state), out.data_ptr(), _stream()))
     return out

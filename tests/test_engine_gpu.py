@@ -336,6 +336,37 @@ def test_sampled_generation_is_batch_invariant(lib, folders):
     assert halves == together
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replay_equals_eager_steps(lib, folders, dtype, tmp_path):
+    """Decode through captured graphs gives the tokens of eager steps: across page borders, when the
+    batch shrinks, when the context outgrows the bound a graph was captured for, and with the
+    program's own eager work (prompts of later batches) between the replays."""
+    from fms_amd.engine import Engine
+    from fms_amd.generation import generate_requests
+    from fms_amd.sampling import SamplingParams
+
+    kw = dict(CONFIGS["A"], max_expected_seq_len=1400)
+    folder = str(tmp_path / "long")
+    lib.write_model_folder(folder, lib.LLaMAConfig(**kw), seed=21, std=0.08, norm_std=0.2)
+    model = lib.get_model("hf_pretrained", model_path=folder, data_type=dtype)
+    prompts = [tokens_for("A", n, 300 + n) for n in (60, 1000, 3, 64, 129)]
+    for params in (SamplingParams(do_sample=False), SamplingParams(do_sample=True, temperature=0.9, top_k=20)):
+        eager = Engine(model, max_tokens=2048, max_slots=3, use_graphs=False)
+        graphs = Engine(model, max_tokens=2048, max_slots=3, use_graphs=True)
+        assert graphs.use_graphs
+        want = generate_requests(eager, prompts, max_new_tokens=70, sampling=params, seed=9, stop_token_ids=[7])
+        got = generate_requests(graphs, prompts, max_new_tokens=70, sampling=params, seed=9, stop_token_ids=[7])
+        if dtype == "float32":
+            assert got == want
+        else:
+            # bfloat16: equal kernels, equal order of operations: equal tokens
+            assert got == want
+        again = generate_requests(graphs, prompts, max_new_tokens=70, sampling=params, seed=9, stop_token_ids=[7])
+        assert again == got  # the graphs captured above are replayed, not captured anew
+        graphs.cache.check()
+        assert graphs.cache.live_slots() == []
+
+
 # --------------------------------------------------------------------------
 def run_trace(folder, dtype, steps, out_dir, max_tokens):
     proc = subprocess.Popen(
