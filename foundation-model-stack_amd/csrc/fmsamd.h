@@ -87,10 +87,6 @@ int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* 
 int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                   int out_dtype, long ldo, int M, int hidden, int K, int act, hipStream_t stream);
 
-// tuning aid: the skinny product (M <= 16, bfloat16 out) with explicit launch shape
-int fmsamd_gemm_skinny_variant(const void* x, long ldx, const void* w, void* out, long ldo, int M, int N, int K,
-                               int waves, int unr, int ntb, hipStream_t stream);
-
 // token choice; rng_state is [rows][2] uint64 (seed, counter), advanced by the kernel
 int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature, int top_k,
                   void* rng_state, int* out_tokens, hipStream_t stream);

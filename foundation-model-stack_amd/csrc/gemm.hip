@@ -374,25 +374,3 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
   FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
   return 0;
 }
-
-// Tuning aid: the plain skinny product (M <= 16, bfloat16 out, no bias) with an explicit choice of
-// waves per block, chunks in flight per wave and tiles per block.
-template <int W, int U, int NTB>
-static void launch_variant(const void* x, long ldx, const void* w, void* out, long ldo, int M, int N, int K,
-                           hipStream_t stream) {
-  const int blocks = ceil_div(N, 16 * NTB);
-  skinny_bf16_kernel<W, U, NTB, 1, false, bf16, bf16><<<blocks, W * WAVE, 0, stream>>>(
-      (const bf16*)x, ldx, (const bf16*)w, (const bf16*)nullptr, (bf16*)out, ldo, M, N, K, 0, 0);
-}
-
-extern "C" int fmsamd_gemm_skinny_variant(const void* x, long ldx, const void* w, void* out, long ldo, int M, int N,
-                                          int K, int waves, int unr, int ntb, hipStream_t stream) {
-  FMS_REQUIRE(M > 0 && M <= 16 && N > 0 && K > 0 && K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_variant: bad sizes");
-#define FMS_V(W, U, T) \
-  if (waves == W && unr == U && ntb == T) { launch_variant<W, U, T>(x, ldx, w, out, ldo, M, N, K, stream); FMS_LAUNCH_CHECK("gemm_skinny_variant"); return 0; }
-  FMS_V(4, 1, 1) FMS_V(4, 2, 1) FMS_V(4, 4, 1) FMS_V(4, 8, 1) FMS_V(8, 1, 1) FMS_V(8, 2, 1) FMS_V(8, 4, 1) FMS_V(8, 8, 1)
-  FMS_V(16, 1, 1) FMS_V(16, 2, 1) FMS_V(16, 4, 1) FMS_V(16, 8, 1)
-  FMS_V(4, 1, 2) FMS_V(4, 2, 2) FMS_V(4, 4, 2) FMS_V(8, 1, 2) FMS_V(8, 2, 2) FMS_V(8, 4, 2) FMS_V(16, 1, 2) FMS_V(16, 2, 2) FMS_V(16, 4, 2)
-#undef FMS_V
-  FMS_REQUIRE(false, "gemm_skinny_variant: no variant waves=%d unr=%d ntb=%d", waves, unr, ntb);
-}

@@ -40,7 +40,6 @@ _SIGNATURES = {
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
     "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
     "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P],
-    "fmsamd_gemm_skinny_variant": [P, L, P, P, L, I, I, I, I, I, I, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
 }
