@@ -1,0 +1,303 @@
+"""Each part alone against its plain formula, and parts the library has never heard of:
+a toy mixer with state of its own, defined here, registered, built into a model through the
+ordinary registries and stepped by the ordinary engine, without touching the library's files."""
+
+import dataclasses
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import plain_llama as P  # noqa: E402
+
+
+@pytest.fixture(scope="module")
+def lib():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import fms_amd
+    from fms_amd.kernels import load
+
+    load()
+    return fms_amd
+
+
+DEV = "cuda"
+
+
+def bind_random(part, dtype, seed=0, std=0.2):
+    """Random tensors for every declared parameter of a part; returns them as float32 CPU tensors by name."""
+    g = torch.Generator().manual_seed(seed)
+    values = {}
+    for name, spec, owner, local in part.named_specs():
+        t = torch.randn(spec.shape, generator=g) * std
+        if spec.init == "ones":
+            t = t + 1
+        t = t.to(dtype)
+        owner.bind(local, t.to(DEV))
+        values[name] = t.float()
+    for p in part.walk():
+        p.finalize(torch.device(DEV), dtype)
+    return values
+
+
+def tol(dtype):
+    return dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=3e-2, rtol=3e-2)
+
+
+def close(got, want, dtype):
+    """float32: element by element; bfloat16: within 3 % of the largest value."""
+    if dtype == torch.float32:
+        torch.testing.assert_close(got, want, atol=1e-4, rtol=1e-4)
+    else:
+        err, scale = float((got - want).abs().max()), float(want.abs().max())
+        assert err <= 0.03 * scale, f"differs by {err:.4g} at a scale of {scale:.4g}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(lib, dtype):
+    from fms_amd.parts import make_part
+
+    norm = make_part("norm", "rmsnorm", width=72, eps=1e-3)
+    w = bind_random(norm, dtype)
+    x = torch.randn(6, 72)
+    branch = torch.randn(6, 72).to(dtype)
+    resid = x.clone().to(DEV)
+    out = norm.add_norm(resid, branch.to(DEV), dtype)
+    torch.testing.assert_close(resid.cpu(), x + branch.float())
+    torch.testing.assert_close(out.cpu().float(), P.rms_norm(x + branch.float(), w["weight"], 1e-3), **tol(dtype))
+
+
+def test_rotary_part(lib):
+    from fms_amd.parts import make_part
+
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 64}
+    rope = make_part("position", "rope", dim=48, theta=50000.0, max_seq_len=300, scaling=scaling)
+    rope.finalize(torch.device(DEV), torch.float32)
+    cos, sin, rot = rope.rotary_tables()
+    assert rot == 48 and cos.shape == (300, 24)
+    freqs = P.rope_frequencies(48, 50000.0, scaling)
+    angles = torch.outer(torch.arange(300).float(), freqs)
+    torch.testing.assert_close(cos.cpu(), torch.cos(angles), atol=2e-6, rtol=0)
+    torch.testing.assert_close(sin.cpu(), torch.sin(angles), atol=2e-6, rtol=0)
+    rope.check_positions(299)
+    with pytest.raises(IndexError):  # tests/modules/test_positions.py:156-168
+        rope.check_positions(300)
+    half = make_part("position", "rope", dim=32, theta=1e4, max_seq_len=16, partial_rope=0.5)
+    assert half.rot_dim == 16
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows", [3, 100])
+def test_feed_forward_part(lib, dtype, rows):
+    from fms_amd.parts import make_part
+
+    ff = make_part("feed_forward", "glu", width=40, hidden_dim=72, activation="swish", use_bias=True)
+    w = bind_random(ff, dtype, seed=1)
+    x = torch.randn(rows, 40).to(dtype)
+    out = ff.forward(x.to(DEV)).cpu().float()
+    want = P.gated_feed_forward(x.float(), w["wg1_fused.weight"], w["w2.weight"], w["wg1_fused.bias"], w["w2.bias"])
+    torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=0.1, rtol=5e-2)))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (3, 1, 32)])
+def test_attention_part_prefill_then_decode(lib, dtype, H, K, D):
+    from fms_amd.cache import KVNeed, SequenceCache
+    from fms_amd.engine.batch import build_batch
+    from fms_amd.kernels import ops
+    from fms_amd.parts import LayerCache, make_part
+
+    width = H * D  # the plain block takes the head size as width / heads
+    rope = make_part("position", "rope", dim=D, theta=1e4, max_seq_len=512)
+    attn = make_part("mixer", "attention", width=width, nheads=H, kvheads=K, head_dim=D, use_bias=True, position_encoder=rope)
+    w = bind_random(attn, dtype, seed=2, std=0.1)
+    rope.finalize(torch.device(DEV), dtype)
+    assert attn.kv_need() == KVNeed(K, D, 0) and attn.state_need() is None
+    cache = SequenceCache([(0, attn.kv_need())], [], max_tokens=1024, max_slots=3, max_seq_len=512, dtype=dtype, device=DEV)
+    lens = [70, 5]
+    xs = [torch.randn(n + 3, width).to(dtype) for n in lens]
+    slots = [cache.alloc_slot() for _ in lens]
+    cfg = P.PlainConfig(vocab=1, width=width, nheads=H, kvheads=K, nlayers=1, hidden=1, eps=0, theta=1e4, max_len=512)
+    freqs = P.rope_frequencies(D, 1e4)
+    want = [P.attention_block(x.float(), torch.arange(x.shape[0]), cfg, w["in_proj.qkv_fused.weight"], w["dense.weight"],
+                              freqs, w["in_proj.qkv_fused.bias"], w["dense.bias"]) for x in xs]
+    group, keys, values = cache.kv_of_entry(0)
+    view = LayerCache(group, keys, values, True, {})
+    # prompts in one step
+    starts = [cache.extend(s, n) for s, n in zip(slots, lens)]
+    batch = build_batch(cache, slots, [[0] * n for n in lens], starts, [[] for _ in lens], DEV, ops.prefill_qblock())
+    out = attn.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).to(DEV), batch, view).cpu().float()
+    close(out, torch.cat([wt[:n] for wt, n in zip(want, lens)]), dtype)
+    # three more tokens each, one at a time
+    for i in range(3):
+        starts = [cache.extend(s, 1) for s in slots]
+        batch = build_batch(cache, slots, [[0], [0]], starts, [[], []], DEV, ops.prefill_qblock())
+        out = attn.forward(torch.stack([x[n + i] for x, n in zip(xs, lens)]).to(DEV), batch, view).cpu().float()
+        close(out, torch.stack([wt[n + i] for wt, n in zip(want, lens)]), dtype)
+
+
+# --------------------------------------------------------------------------
+# parts the library does not have
+# --------------------------------------------------------------------------
+def test_a_toy_mixer_with_state_of_its_own(lib):
+    """A mixer that keeps a running sum per sequence (state of fixed size, no keys or values):
+    y_t = W * mean(x_0..x_t).  It is registered here, chosen by a configuration for some layers of a
+    model whose other layers are attention, built by get_model, stepped by Engine in ragged batches
+    with slots that are used again, and compared with a plain computation."""
+    import fms_amd
+    from fms_amd.architectures import Architecture, register_architecture, register_model
+    from fms_amd.cache import StateNeed
+    from fms_amd.config import ModelConfig
+    from fms_amd.engine import Engine
+    from fms_amd.parts import LayerSpec, Mixer, ModelSpec, PartSpec, ScheduleEntry, register_part, unregister_part
+
+    class RunningMean(Mixer):
+        graph_safe = False  # loops over sequences on the host
+
+        def __init__(self, width, position_encoder=None):
+            super().__init__()
+            self.width = width
+            self.declare("proj.weight", (width, width))
+
+        def state_need(self):
+            return StateNeed((("sum", (self.width,), "float32"), ("count", (1,), "float32")))
+
+        def forward(self, x, batch, cache):
+            total, count = cache.state["sum"], cache.state["count"]
+            out = torch.empty_like(x)
+            at = 0
+            for slot, n in zip(batch.slots, batch.q_lens):
+                xs = x[at : at + n].float()
+                sums = torch.cumsum(xs, 0) + total[slot]
+                counts = count[slot] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+                out[at : at + n] = ((sums / counts[:, None]) @ self.w["proj.weight"].float().t()).to(x.dtype)
+                total[slot] = sums[-1]
+                count[slot] += n
+                at += n
+            return out
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        vocab: int = 90
+        width: int = 48
+        hidden: int = 64
+        max_len: int = 256
+
+    def toy_spec(c: ToyConfig) -> ModelSpec:
+        norm = PartSpec("rmsnorm", {"eps": 1e-5})
+        ff = PartSpec("glu", {"hidden_dim": c.hidden, "activation": "swish"})
+        mean_layer = LayerSpec(mixer=PartSpec("running_mean"), feed_forward=ff, norm=norm)
+        attn_layer = LayerSpec(mixer=PartSpec("attention", {"nheads": 3, "kvheads": 1, "head_dim": 16}), feed_forward=ff,
+                               norm=norm, position="rope")
+        return ModelSpec(vocab=c.vocab, width=c.width, max_seq_len=c.max_len, layers=[mean_layer, attn_layer],
+                         final_norm=norm, positions={"rope": PartSpec("rope", {"dim": 16, "theta": 1e4, "max_seq_len": c.max_len})},
+                         # layer 0 runs twice (two states of its own), layer 1 in between
+                         schedule=[ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)])
+
+    register_part("mixer", "running_mean", RunningMean)
+    try:
+        try:
+            register_architecture(Architecture("toy_running_mean", ToyConfig, toy_spec))
+            register_model("toy_running_mean", "tiny", lambda **kw: ToyConfig().updated(**kw))
+        except KeyError:
+            pass  # a second run in one process
+        model = fms_amd.get_model("toy_running_mean", "tiny", data_type="float32", random_seed=3)
+        kv, state = model.cache_needs()
+        assert [e for e, _ in kv] == [1] and [e for e, _ in state] == [0, 2]
+        engine = Engine(model, max_tokens=512, max_slots=2)
+        assert not engine.use_graphs  # the toy part cannot be captured, so steps run eagerly
+
+        w = {name: owner.w[local].float().cpu() for name, _, owner, local in model.named_specs()}
+
+        def plain(ids):
+            x = w["base_model.embedding.weight"][torch.tensor(ids)]
+            pos = torch.arange(len(ids))
+            cfg = P.PlainConfig(vocab=90, width=48, nheads=3, kvheads=1, nlayers=2, hidden=64, eps=1e-5, theta=1e4, max_len=256)
+            for layer in (0, 1, 0):
+                p = f"base_model.layers.{layer}."
+                h = P.rms_norm(x, w[p + "ln.weight"], 1e-5)
+                if layer == 0:
+                    mean = torch.cumsum(h, 0) / torch.arange(1, len(ids) + 1)[:, None]
+                    h = mean @ w[p + "attn.proj.weight"].t()
+                else:
+                    h = P.attention_block(h, pos, cfg, w[p + "attn.in_proj.qkv_fused.weight"], w[p + "attn.dense.weight"],
+                                          P.rope_frequencies(16, 1e4))
+                x = x + h
+                h = P.rms_norm(x, w[p + "ff_ln.weight"], 1e-5)
+                x = x + P.gated_feed_forward(h, w[p + "ff_sub_layer.wg1_fused.weight"], w[p + "ff_sub_layer.w2.weight"])
+            return P.rms_norm(x, w["base_model.dec_norm.weight"], 1e-5) @ w["head.weight"].t()
+
+        g = torch.Generator().manual_seed(1)
+        for round_ in range(2):  # the second round uses the slots again: their state must start at zero
+            seqs = [torch.randint(0, 90, (n,), generator=g).tolist() for n in (30, 9)]
+            slots = [engine.new_sequence() for _ in seqs]
+            got = [[], []]
+            logits = engine.step(slots, [s[:-4] for s in seqs], "all")
+            got[0].append(logits[: len(seqs[0]) - 4])
+            got[1].append(logits[len(seqs[0]) - 4 :])
+            for i in range(4, 0, -1):
+                logits = engine.step(slots, [[s[-i]] for s in seqs], "last")
+                got[0].append(logits[0:1])
+                got[1].append(logits[1:2])
+            for s in slots:
+                engine.end_sequence(s)
+            for ids, rows in zip(seqs, got):
+                torch.testing.assert_close(torch.cat(rows).cpu(), plain(ids), atol=2e-4, rtol=1e-3)
+        engine.cache.check()
+    finally:
+        unregister_part("mixer", "running_mean")
+
+
+def test_a_layer_named_twice_and_a_layer_reading_another_cache(lib, tmp_path):
+    """The order of layers is data: Llama's own layers in the order 0, 1, 0, with the last entry
+    reading the keys and values that the first one cached (it computes queries only)."""
+    import fms_amd
+    from fms_amd.architectures.llama import llama_spec
+    from fms_amd.engine import Engine
+    from fms_amd.engine.model import DecoderModel
+    from fms_amd.parts import ScheduleEntry
+    from fms_amd.weights import init_random
+
+    config = fms_amd.LLaMAConfig(src_vocab_size=70, emb_dim=64, nheads=4, kvheads=2, nlayers=2, hidden_dim=96, multiple_of=1,
+                                 max_expected_seq_len=256)
+    spec = llama_spec(config)
+    spec.schedule = [ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0, cache_of=0)]
+    model = DecoderModel(spec, torch.float32, config=config)
+    init_random(model, 5, torch.device(DEV), std=0.1, norm_std=0.1)
+    model.finalize_all(DEV)
+    engine = Engine(model, max_tokens=256, max_slots=1)
+    w = {name: owner.w[local].float().cpu() for name, _, owner, local in model.named_specs()}
+    cfg = P.PlainConfig(vocab=70, width=64, nheads=4, kvheads=2, nlayers=2, hidden=96, eps=1e-5, theta=1e4, max_len=256)
+    ids = torch.randint(0, 70, (80,), generator=torch.Generator().manual_seed(2)).tolist()
+
+    def plain(ids):
+        S = len(ids)
+        pos = torch.arange(S)
+        freqs = P.rope_frequencies(16, 1e4)
+        x = w["base_model.embedding.weight"][torch.tensor(ids)]
+        kept = None
+        for n, layer in enumerate((0, 1, 0)):
+            p = f"base_model.layers.{layer}."
+            h = P.rms_norm(x, w[p + "ln.weight"], 1e-5)
+            qkv = h @ w[p + "attn.in_proj.qkv_fused.weight"].t()
+            q, k, v = torch.split(qkv, [64, 32, 32], dim=-1)
+            q = P.rope_rotate(q.reshape(S, 4, 16), pos, freqs)
+            k = P.rope_rotate(k.reshape(S, 2, 16), pos, freqs)
+            v = v.reshape(S, 2, 16)
+            if n == 0:
+                kept = (k, v)
+            if n == 2:
+                k, v = kept  # reads the first entry's cache
+            a = P.causal_attention(q, k, v).reshape(S, 64) @ w[p + "attn.dense.weight"].t()
+            x = x + a
+            h = P.rms_norm(x, w[p + "ff_ln.weight"], 1e-5)
+            x = x + P.gated_feed_forward(h, w[p + "ff_sub_layer.wg1_fused.weight"], w[p + "ff_sub_layer.w2.weight"])
+        return P.rms_norm(x, w["base_model.dec_norm.weight"], 1e-5) @ w["head.weight"].t()
+
+    slot = engine.new_sequence()
+    got = [engine.step([slot], [ids[:70]], "all")] + [engine.step([slot], [[t]], "last") for t in ids[70:]]
+    torch.testing.assert_close(torch.cat(got).cpu(), plain(ids), atol=2e-4, rtol=1e-3)
