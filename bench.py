@@ -35,6 +35,8 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--skip-points", action="store_true", help="leave out decode at batch 1 and 64")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="run one phase only (for profiling); the record then lacks the other")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this library runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -109,11 +111,15 @@ def main() -> int:
         flops += 2.0 * E * V  # the head for one row
         return n_tokens / t, 1000 * t, flops / t / PEAK_FLOPS["bf16"]
 
-    pre_tps, pre_ms, pre_frac = prefill(args.prefill_tokens)
-    tps, ms, step_bytes = decode(args.batch, args.steps, args.warmup)
-    achieved = step_bytes / (ms / 1000) / 1e9
+    pre_tps = pre_ms = pre_frac = 0.0
+    tps = ms = step_bytes = 0.0
+    if args.only != "decode":
+        pre_tps, pre_ms, pre_frac = prefill(args.prefill_tokens)
+    if args.only != "prefill":
+        tps, ms, step_bytes = decode(args.batch, args.steps, args.warmup)
+    achieved = step_bytes / (ms / 1000) / 1e9 if ms else 0.0
     points = {}
-    if not args.skip_points:
+    if not args.skip_points and args.only is None:
         points["decode_b1"] = round(decode(1, min(args.steps, 32), 4)[0], 1)
         points["decode_b64"] = round(decode(64, min(args.steps, 16), 2)[0], 1)
 

@@ -373,29 +373,34 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
   }
 }
 
-template <int MAXDT>
-__global__ void __launch_bounds__(WAVE)
+// Grid (split, kv head x head tile, token).  The waves of a block take the pages of its split in turn and
+// meet in LDS, so that a context of up to waves x pages_per_wave pages needs no second kernel.
+template <int MAXDT, int MAXW>
+__global__ void __launch_bounds__(MAXW* WAVE)
     attn_decode_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                             float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                            int window, int pages_per_split) {
+                            int window, int pages_per_split, int tile_cols) {
+  extern __shared__ float lds[];  // [wave][tile_cols columns][head_dim + 2]
   const int split = blockIdx.x;
   const int group = nheads / kvheads;
-  const int tiles_per_kv = (group + 15) / 16;
+  const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
   const int kh = blockIdx.y / tiles_per_kv;
   const int ht = blockIdx.y % tiles_per_kv;
   const int t = blockIdx.z;
-  const int lane = threadIdx.x;
+  const int wave = threadIdx.x / WAVE;
+  const int n_waves = blockDim.x / WAVE;
+  const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
   const int seq = seq_of_token[t];
-  const int cols = group - ht * 16 < 16 ? group - ht * 16 : 16;  // query heads in this tile
-  const int head0 = kh * group + ht * 16;
+  const int cols = group - ht * tile_cols < tile_cols ? group - ht * tile_cols : tile_cols;  // query heads here
+  const int head0 = kh * group + ht * tile_cols;
   if (seq < 0) {
     if (split == 0)
-      for (int i = lane; i < cols * head_dim; i += WAVE)
+      for (int i = threadIdx.x; i < cols * head_dim; i += blockDim.x)
         out[(size_t)t * out_stride + (size_t)head0 * head_dim + i] = (bf16)0.f;
     return;
   }
@@ -418,7 +423,7 @@ __global__ void __launch_bounds__(WAVE)
 
   WaveState<MAXDT, 1> st;
   wave_state_init(st);
-  for (int pi = page_lo; pi <= page_hi; ++pi) {
+  for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
     const size_t phys = (size_t)bt[pi];
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
@@ -430,32 +435,47 @@ __global__ void __launch_bounds__(WAVE)
     }
   }
 
+  // ---- the waves of the block meet in LDS --------------------------------
   const int ndt = head_dim / 16;
+  const int cstride = head_dim + 2;
   float l = st.l[0];
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
-  if (r >= cols) return;
-  const int head = head0 + r;
-  if (n_splits == 1) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    bf16* orow = out + (size_t)t * out_stride + (size_t)head * head_dim;
-#pragma unroll
-    for (int dt = 0; dt < MAXDT; ++dt) {
-      if (dt < ndt) {
-        const f32x4 a = st.acc[0][dt];
-        const bf16x4 o = {(bf16)(a[0] * inv), (bf16)(a[1] * inv), (bf16)(a[2] * inv), (bf16)(a[3] * inv)};
-        *reinterpret_cast<bf16x4*>(orow + dt * 16 + g * 4) = o;
-      }
+  if (r < cols) {
+    float* dst = lds + ((size_t)wave * tile_cols + r) * cstride;
+    if (g == 0) {
+      dst[head_dim] = st.m[0];
+      dst[head_dim + 1] = l;
     }
-  } else {
-    const size_t base = ((size_t)t * nheads + head) * n_splits + split;
-    float* prow = part_o + base * head_dim;
 #pragma unroll
     for (int dt = 0; dt < MAXDT; ++dt)
-      if (dt < ndt) *reinterpret_cast<f32x4*>(prow + dt * 16 + g * 4) = st.acc[0][dt];
-    if (g == 0) {
-      part_ml[base * 2] = st.m[0];
-      part_ml[base * 2 + 1] = l;
+      if (dt < ndt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dst[dt * 16 + g * 4 + i] = st.acc[0][dt][i];
+  }
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < cols * head_dim; idx += blockDim.x) {
+    const int c = idx / head_dim;
+    const int d = idx % head_dim;
+    float m = -1e30f;
+    for (int w = 0; w < n_waves; ++w) m = fmaxf(m, lds[((size_t)w * tile_cols + c) * cstride + head_dim]);
+    float o = 0.f, lsum = 0.f;
+    for (int w = 0; w < n_waves; ++w) {
+      const float* src = lds + ((size_t)w * tile_cols + c) * cstride;
+      const float f = __expf(src[head_dim] - m);
+      o += f * src[d];
+      lsum += f * src[head_dim + 1];
+    }
+    const int head = head0 + c;
+    if (n_splits == 1) {
+      out[(size_t)t * out_stride + (size_t)head * head_dim + d] = (bf16)(lsum > 0.f ? o / lsum : 0.f);
+    } else {
+      const size_t base = ((size_t)t * nheads + head) * n_splits + split;
+      part_o[base * head_dim + d] = o;
+      if (d == 0) {
+        part_ml[base * 2] = m;
+        part_ml[base * 2 + 1] = lsum;
+      }
     }
   }
 }
@@ -559,35 +579,41 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        long workspace_bytes, const int* positions, const int* seq_of_token,
                                        const int* block_table, int table_stride, const void* k_cache,
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
-                                       float scale, int window, int max_context, int pages_per_split,
+                                       float scale, int window, int max_context, int pages_per_split, int waves,
                                        hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
-  FMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attn_decode_bf16: row strides must keep 16-byte alignment");
+  FMS_REQUIRE(q_stride % 8 == 0, "attn_decode_bf16: query row stride must keep 16-byte alignment");
   FMS_REQUIRE(pages_per_split > 0 && max_context > 0, "attn_decode_bf16: bad split sizes");
+  FMS_REQUIRE(waves >= 1 && waves <= 8, "attn_decode_bf16: %d waves per block (1..8)", waves);
+  if (head_dim > 128 && waves > 4) waves = 4;
   FMS_REQUIRE(n_tokens <= 65535, "attn_decode_bf16: %d tokens exceed one launch (65535)", n_tokens);
   const int n_splits = ceil_div(ceil_div(max_context, PAGE_TOKENS), pages_per_split);
   const long need = fmsamd_attn_decode_workspace(n_tokens, nheads, head_dim, n_splits);
   FMS_REQUIRE(workspace_bytes >= need, "attn_decode_bf16: workspace of %ld bytes, %ld needed", workspace_bytes, need);
-  FMS_REQUIRE(need == 0 || ((size_t)workspace % 16) == 0, "attn_decode_bf16: workspace must be 16-byte aligned");
   const int group = nheads / kvheads;
-  const int tiles_per_kv = (group + 15) / 16;
+  // the merge buffer [waves][columns][head_dim + 2] must fit 64 KB of LDS
+  int tile_cols = 16;
+  while (tile_cols > 1 && (size_t)waves * tile_cols * (head_dim + 2) * sizeof(float) > 65536) tile_cols /= 2;
+  const size_t lds_bytes = (size_t)waves * tile_cols * (head_dim + 2) * sizeof(float);
+  FMS_REQUIRE(lds_bytes <= 65536, "attn_decode_bf16: %d waves need %zu bytes of LDS", waves, lds_bytes);
+  const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
   FMS_REQUIRE((long)kvheads * tiles_per_kv <= 65535, "attn_decode_bf16: too many heads");
   float* part_o = (float*)workspace;
   float* part_ml = part_o ? part_o + (size_t)n_tokens * nheads * n_splits * head_dim : nullptr;
   dim3 grid(n_splits, kvheads * tiles_per_kv, n_tokens);
-#define FMS_DC(M)                                                                                                    \
-  attn_decode_bf16_kernel<M><<<grid, dim3(WAVE), 0, stream>>>(                                                       \
+#define FMS_DC(M, MAXW)                                                                                              \
+  attn_decode_bf16_kernel<M, MAXW><<<grid, dim3(waves * WAVE), lds_bytes, stream>>>(                                 \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, pages_per_split)
+      window, pages_per_split, tile_cols)
   if (head_dim <= 64)
-    FMS_DC(4);
+    FMS_DC(4, 8);
   else if (head_dim <= 128)
-    FMS_DC(8);
+    FMS_DC(8, 8);
   else
-    FMS_DC(16);
+    FMS_DC(16, 4);  // large heads need the registers of a smaller block
 #undef FMS_DC
   FMS_LAUNCH_CHECK("attn_decode_bf16");
   if (n_splits > 1) {

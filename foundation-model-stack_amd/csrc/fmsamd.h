@@ -69,13 +69,14 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                              hipStream_t stream);
 
-// bfloat16 decode: one token per sequence, keys split over one-wave blocks of `pages_per_split` pages
+// bfloat16 decode: one token per sequence.  A block of `waves` waves covers `pages_per_split` pages (its waves
+// take them in turn and merge in LDS); with more than one split a second kernel merges the partial results.
 long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits);
 int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_stride, void* workspace,
                             long workspace_bytes, const int* positions, const int* seq_of_token,
                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
-                            int max_context, int pages_per_split, hipStream_t stream);
+                            int max_context, int pages_per_split, int waves, hipStream_t stream);
 
 // c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
 int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,
@@ -86,6 +87,14 @@ int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* 
                             int out_dtype, long ldo, int M, int N, int K, hipStream_t stream);
 int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                   int out_dtype, long ldo, int M, int hidden, int K, int act, hipStream_t stream);
+
+// qkv = x W^T (+ bias) for at most 32 rows with the rotation and the cache write fused into the epilogue;
+// only the query columns of `out` are written
+int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
+                                long ldo, int M, int K, const int* positions, const int* seq_of_token,
+                                const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
+                                int rot_dim, int max_pos, void* k_cache, void* v_cache, int nheads, int kvheads,
+                                int head_dim, hipStream_t stream);
 
 // token choice; rng_state is [rows][2] uint64 (seed, counter), advanced by the kernel
 int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature, int top_k,

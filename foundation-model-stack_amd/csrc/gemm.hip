@@ -198,21 +198,54 @@ __device__ __forceinline__ float sk_activate(float x, int kind) {
   }
 }
 
+// What the skinny kernel does with a finished output element.
+#define EPI_PLAIN 0  // store (+ bias)
+#define EPI_GATED 1  // the block's second tile is the "up" half: out = act(first) * second, N is the hidden size
+#define EPI_ROPE 2   // the output row is [queries | keys | values] of attention: rotate q and k, store q, and
+                     // write k and v into their cache pages (layout: see rope.hip)
+
+struct RopeEpilogue {
+  const int* positions;     // [M]
+  const int* seq_of_token;  // [M], -1: padding row
+  const int* block_table;
+  int table_stride;
+  const float* cos_t;  // [max_pos, rot_dim/2] or null
+  const float* sin_t;
+  int rot_dim, max_pos;
+  bf16* k_cache;  // null: queries only
+  bf16* v_cache;
+  int nheads, kvheads, head_dim;
+};
+
 // NTB: 16-row tiles of W per block (the second tile starts `tile2_offset` rows after the first).
 // MT : 16-row tiles of x.
-// GATED: the second tile is the "up" half; out = act(first) * second, N is the hidden size.
 // SK_WAVES: waves of a block (8, or 4 when NTB*MT > 4 so that the LDS buffer stays under 64 KB).
 // UNR: chunks of 64 k-values whose loads a wave issues before it multiplies: what keeps enough
 // bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 2 loads of 16 bytes outstanding).
-template <int SK_WAVES, int UNR, int NTB, int MT, bool GATED, typename OutT, typename BiasT>
+template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typename BiasT>
 __global__ void __launch_bounds__(SK_WAVES* WAVE)
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
-                       OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act) {
+                       OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
+                       RopeEpilogue rope) {
+  constexpr bool GATED = EPI == EPI_GATED;
   __shared__ float red[SK_WAVES][NTB][MT][16][17];
+  __shared__ int s_pos[MT * 16], s_seq[MT * 16], s_page[MT * 16];
   const int wave = threadIdx.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
   const int n0 = blockIdx.x * 16 * (GATED ? 1 : NTB);
+
+  if (EPI == EPI_ROPE && threadIdx.x < MT * 16) {
+    // index data of the rows, fetched while the weights stream
+    const int m = threadIdx.x;
+    int pos = 0, seq = -1, page = 0;
+    if (m < M) {
+      seq = rope.seq_of_token[m];
+      pos = rope.positions[m];
+      if (seq >= 0 && rope.k_cache) page = rope.block_table[(size_t)seq * rope.table_stride + pos / PAGE_TOKENS];
+    }
+    s_pos[m] = pos, s_seq[m] = seq, s_page[m] = page;
+  }
 
   const bf16* wrow[NTB];
   bool wok[NTB];
@@ -278,6 +311,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
   __syncthreads();
 
   constexpr int OUT_TILES = GATED ? 1 : NTB;
+  // every thread of a wave runs the same number of rounds (the rotation reads its neighbour's value)
   for (int idx = threadIdx.x; idx < OUT_TILES * MT * 256; idx += blockDim.x) {
     const int nn = idx & 15;           // n within tile: fastest, so that stores of a row are contiguous
     const int mm = (idx >> 4) & 15;    // m within tile
@@ -285,11 +319,12 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
     const int ti = (idx >> 8) / MT;    // n tile
     const int m = tj * 16 + mm;
     const int n = n0 + ti * 16 + nn;
-    if (m >= M || n >= N) continue;
+    const bool live = m < M && n < N;
     float v = 0.f;
 #pragma unroll
     for (int wv = 0; wv < SK_WAVES; ++wv) v += red[wv][ti][tj][nn][mm];
-    if (GATED) {
+    if (EPI == EPI_GATED) {
+      if (!live) continue;
       float u = 0.f;
 #pragma unroll
       for (int wv = 0; wv < SK_WAVES; ++wv) u += red[wv][1][tj][nn][mm];
@@ -297,30 +332,57 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
         v += to_f32(bias[n]);
         u += to_f32(bias[tile2_offset + n]);
       }
-      v = sk_activate(v, act) * u;
-    } else if (bias) {
-      v += to_f32(bias[n]);
+      out[(size_t)m * ldo + n] = from_f32<OutT>(sk_activate(v, act) * u);
+    } else if (EPI == EPI_ROPE) {
+      if (bias && live) v += to_f32(bias[n]);
+      const float partner = __shfl_xor(v, 1, WAVE);  // the other element of the rotary pair: N is a multiple of 16
+      if (!live) continue;
+      const int D = rope.head_dim;
+      const int hh = n / D, d = n - hh * D;
+      const int pos = s_pos[m], seq = s_seq[m];
+      if (hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr && d < rope.rot_dim) {
+        const int tpos = pos < rope.max_pos ? pos : rope.max_pos - 1;  // the host has checked the range
+        const float c = rope.cos_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
+        const float sn = rope.sin_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
+        v = (d & 1) ? sn * partner + c * v : c * v - sn * partner;
+      }
+      if (hh < rope.nheads) {
+        out[(size_t)m * ldo + n] = from_f32<OutT>(v);
+      } else if (seq >= 0 && rope.k_cache != nullptr) {
+        const size_t page_elems = (size_t)rope.kvheads * PAGE_TOKENS * D;
+        const int in_page = pos % PAGE_TOKENS;
+        if (hh < rope.nheads + rope.kvheads) {
+          const int kh = hh - rope.nheads;
+          rope.k_cache[(size_t)s_page[m] * page_elems + ((size_t)kh * PAGE_TOKENS + in_page) * D + d] = (bf16)v;
+        } else {
+          const int kh = hh - rope.nheads - rope.kvheads;
+          rope.v_cache[(size_t)s_page[m] * page_elems + ((size_t)kh * D + d) * PAGE_TOKENS + in_page] = (bf16)v;
+        }
+      }
+    } else {
+      if (!live) continue;
+      if (bias) v += to_f32(bias[n]);
+      out[(size_t)m * ldo + n] = from_f32<OutT>(v);
     }
-    out[(size_t)m * ldo + n] = from_f32<OutT>(v);
   }
 }
 
-template <int NTB, int MT, bool GATED>
+template <int NTB, int MT, int EPI>
 static void launch_skinny(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                           int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int blocks,
-                          hipStream_t stream) {
+                          hipStream_t stream, RopeEpilogue rope = RopeEpilogue{}) {
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
   constexpr int SK_WAVES = NTB * MT > 4 ? 4 : 8;
   constexpr int UNR = (NTB + MT) <= 2 ? 4 : ((NTB + MT) <= 4 ? 2 : 1);
-#define FMS_SK(O, B)                                                                                  \
-  skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, GATED, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(    \
-      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act)
+#define FMS_SK(O, B)                                                                                 \
+  skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, EPI, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(     \
+      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, rope)
   if (out_dtype == FMS_BF16) {
     if (fb)
       FMS_SK(bf16, float);
     else
       FMS_SK(bf16, bf16);
-  } else {
+  } else if (EPI != EPI_ROPE) {
     if (fb)
       FMS_SK(float, float);
     else
@@ -342,7 +404,7 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   const bool two = N >= 16384;
   const int blocks = ceil_div(N, two ? 32 : 16);
 #define FMS_LS(NTB, MT) \
-  launch_skinny<NTB, MT, false>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, blocks, stream)
+  launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, blocks, stream)
   if (two) {
     if (mt == 1) FMS_LS(2, 1); else if (mt == 2) FMS_LS(2, 2); else if (mt == 3) FMS_LS(2, 3); else FMS_LS(2, 4);
   } else {
@@ -368,9 +430,41 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
   const int mt = ceil_div(M, 16);
   const int blocks = ceil_div(hidden, 16);
 #define FMS_LG(MT) \
-  launch_skinny<2, MT, true>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, blocks, stream)
+  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, blocks, stream)
   if (mt == 1) FMS_LG(1); else if (mt == 2) FMS_LG(2); else if (mt == 3) FMS_LG(3); else FMS_LG(4);
 #undef FMS_LG
   FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
+  return 0;
+}
+
+// qkv[M, (H+2K)*D] = x W^T (+ bias) with the rotation of q and k and the cache write of k and v fused into
+// the epilogue: the decode-time twin of fmsamd_gemm_skinny_bf16 followed by fmsamd_rope_kv_write.  Only the
+// query columns of `out` are written.  M <= 32.
+extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
+                                           void* out, long ldo, int M, int K, const int* positions,
+                                           const int* seq_of_token, const int* block_table, int table_stride,
+                                           const float* cos_t, const float* sin_t, int rot_dim, int max_pos,
+                                           void* k_cache, void* v_cache, int nheads, int kvheads, int head_dim,
+                                           hipStream_t stream) {
+  if (M == 0) return 0;
+  const int N = (nheads + 2 * kvheads) * head_dim;
+  FMS_REQUIRE(M > 0 && M <= 32 && K > 0 && nheads > 0 && kvheads > 0 && head_dim > 0,
+              "qkv_rope_skinny_bf16: bad sizes M=%d K=%d (M <= 32)", M, K);
+  FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "qkv_rope_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
+  FMS_REQUIRE(ldx >= K && ldo >= N, "qkv_rope_skinny_bf16: leading dimensions too small");
+  FMS_REQUIRE(head_dim % 2 == 0 && N % 16 == 0, "qkv_rope_skinny_bf16: head size %d must be even and the row a multiple of 16",
+              head_dim);
+  FMS_REQUIRE(rot_dim % 2 == 0 && rot_dim >= 0 && rot_dim <= head_dim, "qkv_rope_skinny_bf16: rotary size %d does not fit",
+              rot_dim);
+  FMS_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "qkv_rope_skinny_bf16: key and value cache must come together");
+  FMS_REQUIRE(cos_t == nullptr || (max_pos > 0 && sin_t != nullptr), "qkv_rope_skinny_bf16: empty rotary table");
+  RopeEpilogue rope{positions, seq_of_token, block_table, table_stride, rot_dim > 0 ? cos_t : nullptr, sin_t, rot_dim,
+                    max_pos, (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim};
+  const int blocks = N / 16;
+  if (M <= 16)
+    launch_skinny<1, 1, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, rope);
+  else
+    launch_skinny<1, 2, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, rope);
+  FMS_LAUNCH_CHECK("qkv_rope_skinny_bf16");
   return 0;
 }

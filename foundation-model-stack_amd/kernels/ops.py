@@ -184,6 +184,58 @@ def _check_batch_index(positions, seq_of_token, block_table, n_tokens: int) -> N
         raise ValueError("positions and seq_of_token must have an entry per token")
 
 
+def qkv_rope_write(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    positions: torch.Tensor,
+    seq_of_token: torch.Tensor,
+    block_table: torch.Tensor,
+    cos: Optional[torch.Tensor],
+    sin: Optional[torch.Tensor],
+    rot_dim: int,
+    k_cache: Optional[torch.Tensor],
+    v_cache: Optional[torch.Tensor],
+    nheads: int,
+    kvheads: int,
+    head_dim: int,
+) -> torch.Tensor:
+    """The fused qkv projection of a decode step (at most 32 rows, bfloat16): x W^T (+ bias), q and k
+    rotated, k and v written into their cache pages.  Returns the [M, (H+2K)*D] buffer whose query
+    columns hold the rotated queries (its other columns are not written).  Equal to `linear` followed
+    by `rope_kv_write`."""
+    _need_cuda(x, weight, bias, positions, seq_of_token, block_table, cos, sin, k_cache, v_cache)
+    _rows2d("x", x)
+    M, K = x.shape
+    N = (nheads + 2 * kvheads) * head_dim
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or tuple(weight.shape) != (N, K) or not weight.is_contiguous():
+        raise ValueError(f"qkv_rope_write takes bfloat16 x [M, {K}] and a contiguous bfloat16 weight [{N}, {K}]")
+    if M > QKV_ROPE_MAX_ROWS or K % 8 or x.stride(0) % 8 or N % 16:
+        raise ValueError("qkv_rope_write: at most 32 rows, K a multiple of 8, the output row a multiple of 16")
+    if bias is not None and (bias.shape != (N,) or not bias.is_contiguous()):
+        raise ValueError(f"bias must be a contiguous [{N}] tensor")
+    _check_batch_index(positions, seq_of_token, block_table, M)
+    max_pos = 0
+    if cos is not None:
+        if cos.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] * 2 != rot_dim:
+            raise ValueError("cos/sin tables must be float32 [max_pos, rot_dim/2]")
+        if not (cos.is_contiguous() and sin.is_contiguous()):
+            raise ValueError("cos/sin tables must be contiguous")
+        max_pos = cos.shape[0]
+    if k_cache is not None:
+        _check_cache(k_cache, v_cache, kvheads, head_dim, torch.bfloat16)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    check(load().fmsamd_qkv_rope_skinny_bf16(
+        x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
+        out.data_ptr(), out.stride(0), M, K, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
+        block_table.stride(0), _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, max_pos, _ptr(k_cache),
+        _ptr(v_cache), nheads, kvheads, head_dim, _stream()))
+    return out
+
+
+QKV_ROPE_MAX_ROWS = 32
+
+
 def rope_kv_write(
     qkv: torch.Tensor,
     positions: torch.Tensor,
@@ -242,6 +294,7 @@ def attention(
     qblock_start: Optional[torch.Tensor] = None,
     qblock_len: Optional[torch.Tensor] = None,
     pages_per_block: int = 0,
+    waves: int = 0,
     force_generic: bool = False,
 ) -> torch.Tensor:
     """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim].
@@ -269,15 +322,18 @@ def attention(
         if max_context <= 0:
             raise ValueError("decode attention needs max_context (an upper bound of every context length)")
         n_pages = -(-max_context // PAGE_TOKENS)
+        auto_pages, auto_waves = decode_split(T * kvheads, n_pages)
         if pages_per_block <= 0:
-            pages_per_block = decode_pages_per_block(T * kvheads, n_pages)
+            pages_per_block = auto_pages
+        if waves <= 0:
+            waves = min(auto_waves, pages_per_block)
         n_splits = -(-n_pages // pages_per_block)
         ws_bytes = lib.fmsamd_attn_decode_workspace(T, nheads, head_dim, n_splits)
         ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=q.device) if ws_bytes else None
         check(lib.fmsamd_attn_decode_bf16(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _ptr(ws), ws_bytes,
                                           positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), T, nheads, kvheads,
-                                          head_dim, float(scale), int(window), int(max_context), int(pages_per_block), _stream()))
+                                          head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves), _stream()))
         return out
     if qblock_start is None or qblock_len is None:
         raise ValueError("bfloat16 prefill attention needs the query blocks of the batch")
@@ -290,13 +346,15 @@ def attention(
     return out
 
 
-def decode_pages_per_block(rows: int, n_pages: int) -> int:
-    """How many pages one wave of the decode kernel takes: one, unless that would make more than
-    some ten thousand waves or more than 64 partial results per token to merge."""
-    per_split = 1
-    while rows * -(-n_pages // per_split) > 16384 or -(-n_pages // per_split) > 64:
-        per_split *= 2
-    return per_split
+def decode_split(rows: int, n_pages: int):
+    """(pages per split, waves per block) of the decode attention kernel.
+
+    rows = tokens x kv heads.  With 64 rows or more one block per row takes the whole context (its
+    waves share the pages and merge in LDS, no second kernel); fewer rows split the context over
+    several blocks so that the GPU still has some hundred waves to keep the cache in flight."""
+    waves = max(1, min(8, n_pages))
+    splits = 1 if rows >= 64 else min(-(-64 // max(rows, 1)), -(-n_pages // waves))
+    return max(1, -(-n_pages // splits)), waves
 
 
 def prefill_qblock() -> int:

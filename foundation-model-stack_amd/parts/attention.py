@@ -67,16 +67,24 @@ class MultiHeadAttention(Mixer):
 
     def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
         H, K, D = self.nheads, self.kvheads, self.head_dim
-        qkv = self.qkv.forward(x)
         table = batch.block_tables[cache.group]
         tables = self.position_encoder.rotary_tables() if self.position_encoder is not None else None
-        if tables is None and self.position_encoder is not None:
-            self.position_encoder.adjust_qk(qkv, batch, H, K, D)
         cos, sin, rot = tables if tables is not None else (None, None, 0)
-        ops.rope_kv_write(
-            qkv, batch.positions, batch.seq_of_token, table, cos, sin, rot,
-            cache.keys if cache.owns else None, cache.values if cache.owns else None, H, K, D,
+        keys, values = (cache.keys, cache.values) if cache.owns else (None, None)
+        weight = self.qkv.w["weight"]
+        fused = (
+            batch.is_decode and x.shape[0] <= ops.QKV_ROPE_MAX_ROWS and x.dtype == torch.bfloat16
+            and weight.dtype == torch.bfloat16 and D % 16 == 0 and (tables is not None or self.position_encoder is None)
         )
+        if fused:
+            # decode: projection, rotation and cache write in one kernel
+            qkv = ops.qkv_rope_write(x, weight, self.qkv.w.get("bias"), batch.positions, batch.seq_of_token, table,
+                                     cos, sin, rot, keys, values, H, K, D)
+        else:
+            qkv = self.qkv.forward(x)
+            if tables is None and self.position_encoder is not None:
+                self.position_encoder.adjust_qk(qkv, batch, H, K, D)
+            ops.rope_kv_write(qkv, batch.positions, batch.seq_of_token, table, cos, sin, rot, keys, values, H, K, D)
         mixed = ops.attention(
             qkv, batch.positions, batch.seq_of_token, table, cache.keys, cache.values, H, K, D, self.scale, self.window,
             decode=batch.is_decode, max_context=batch.max_context,

@@ -185,6 +185,45 @@ def test_rope_kv_write(ops, dtype, H, K, D, rot):
             assert float(kc[p].abs().sum()) == 0 and float(vc[p].abs().sum()) == 0
 
 
+@pytest.mark.parametrize("M", [1, 8, 20, 32])
+@pytest.mark.parametrize("H,K,D,rot,E", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 40), (8, 8, 32, 16, 256)])
+def test_qkv_rope_write_equals_the_separate_kernels(ops, M, H, K, D, rot, E):
+    """The decode-time fusion (projection + rotation + cache write) against linear followed by rope_kv_write."""
+    torch.manual_seed(11)
+    dtype = torch.bfloat16
+    N = (H + 2 * K) * D
+    x = torch.randn(M, E).to(dtype)
+    w = (torch.randn(N, E) * 0.2).to(dtype)
+    bias = torch.randn(N).to(dtype)
+    positions = torch.randint(0, 200, (M,)).int()
+    seq = torch.arange(M).int()
+    if M > 2:
+        seq[1] = -1  # a padding row: nothing of it may reach the cache
+        seq[2:] -= 1
+    n_seqs = int(seq.max()) + 1
+    table, n_pages = make_pages([256] * n_seqs, K, D, dtype, seed=3)
+    freqs = P.rope_frequencies(rot, 10000.0)
+    cos, sin = ops.rope_table(dev(freqs), 256)
+    for b in (None, bias):
+        caches = []
+        outs = []
+        for fused in (False, True):
+            kc = torch.zeros(n_pages, K, PAGE, D, dtype=dtype, device="cuda")
+            vc = torch.zeros(n_pages, K, D, PAGE, dtype=dtype, device="cuda")
+            args = (dev(positions), dev(seq), dev(table), cos, sin, rot, kc, vc, H, K, D)
+            if fused:
+                qkv = ops.qkv_rope_write(dev(x), dev(w), None if b is None else dev(b), *args)
+            else:
+                qkv = ops.linear(dev(x), dev(w), None if b is None else dev(b))
+                ops.rope_kv_write(qkv, *args)
+            outs.append(qkv[:, : H * D].cpu().float()[seq >= 0])  # a padding row's queries are never read
+            caches.append((kc.cpu().float(), vc.cpu().float()))
+        torch.testing.assert_close(outs[1], outs[0], atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(caches[1][0], caches[0][0], atol=2e-2, rtol=2e-2)
+        torch.testing.assert_close(caches[1][1], caches[0][1], atol=2e-2, rtol=2e-2)
+        assert float(caches[0][0].abs().sum()) > 0
+
+
 # --------------------------------------------------------------------------
 def reference_attention(qs, ks, vs, starts, H, K, scale=None, window=0):
     """qs[b]: [n_b, H, D] queries at positions starts[b]..; ks/vs[b]: [len_b, K, D] all keys."""
@@ -254,8 +293,10 @@ def test_attention_prefill_bf16(ops, H, K, D):
 @pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (8, 2, 128), (2, 2, 64), (40, 2, 32), (2, 1, 256), (5, 5, 80)])
 def test_attention_decode_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 63, 64, 700], lens=[1, 1, 1, 1], decode=True)
-    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=2)
-    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=5)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=2, waves=1)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=5, waves=3)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=24, waves=8)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2, 600], lens=[1, 1, 1], decode=True, pages_per_block=16, waves=4)
 
 
 @pytest.mark.parametrize("dtype,decode", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
