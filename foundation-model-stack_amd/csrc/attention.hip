@@ -93,19 +93,95 @@ struct WaveState {
 __device__ __forceinline__ bf16x8 load_bf16x8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
 __device__ __forceinline__ bf16x4 load_bf16x4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 
+// One step of the online softmax over 32 keys for the 16*QT query columns of a wave.
 // qreg[qt][c]: this lane's 8 query elements d = c*32 + (lane/16)*8 .. +8 of its column (zero when absent).
 // qpos/qlo: visible keys of this lane's column are qlo <= key <= qpos (qpos < 0: no key).
+// kbase: key row 0 of the 32 keys, rows k_stride elements apart; vbase: column 0 of the 32 keys in the
+// transposed values, rows (head_dim of them) v_stride elements apart.  Global memory or LDS.
+template <int MAXDT, int QT>
+__device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
+                                          const int (&qpos)[QT], const int (&qlo)[QT], int key0, const bf16* kbase,
+                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, float scale) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int ndt = head_dim / 16;
+  const int nchunk = (head_dim + 31) / 32;
+  f32x4 sa[QT], sb[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    sa[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    sb[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+#pragma unroll
+  for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
+    if (c < nchunk) {
+      const int d = c * 32 + g * 8;
+      bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0}, kb = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (d < head_dim) {
+        ka = load_bf16x8(kbase + (size_t)r * k_stride + d);
+        kb = load_bf16x8(kbase + (size_t)(16 + r) * k_stride + d);
+      }
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        sa[qt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[qt][c], sa[qt], 0, 0, 0);
+        sb[qt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[qt][c], sb[qt], 0, 0, 0);
+      }
+    }
+  }
+  bf16x8 pmat[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    float mx = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int ja = key0 + g * 4 + i;
+      const int jb = ja + 16;
+      sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale : -INFINITY;
+      sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale : -INFINITY;
+      mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = fmaxf(st.m[qt], mx);
+    const float alpha = __expf(st.m[qt] - m_new);
+    st.m[qt] = m_new;
+    float psum = 0.f;
+    float pa[4], pb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pa[i] = __expf(sa[qt][i] - m_new);
+      pb[i] = __expf(sb[qt][i] - m_new);
+      psum += pa[i] + pb[i];
+    }
+    st.l[qt] = st.l[qt] * alpha + psum;
+    pmat[qt] = bf16x8{(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3],
+                      (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt)
+      if (dt < ndt) st.acc[qt][dt] *= alpha;
+  }
+#pragma unroll
+  for (int dt = 0; dt < MAXDT; ++dt) {
+    if (dt < ndt) {
+      const bf16* vrow = vbase + (size_t)(dt * 16 + r) * v_stride + g * 4;
+      const bf16x4 va = load_bf16x4(vrow);
+      const bf16x4 vb = load_bf16x4(vrow + 16);
+      const bf16x8 v = {va[0], va[1], va[2], va[3], vb[0], vb[1], vb[2], vb[3]};
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt)
+        st.acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat[qt], st.acc[qt][dt], 0, 0, 0);
+    }
+  }
+}
+
+// The pages page_first, page_first + page_step, ... of a sequence, straight from global memory.
 template <int MAXDT, int QT>
 __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
                                                 const int (&qpos)[QT], const int (&qlo)[QT], int key_lo, int key_hi,
                                                 int page_first, int page_step, const int* __restrict__ bt,
                                                 const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
                                                 size_t page_elems, int kh, int head_dim, float scale) {
-  const int lane = threadIdx.x & (WAVE - 1);
-  const int r = lane & 15;
-  const int g = lane >> 4;
-  const int ndt = head_dim / 16;
-  const int nchunk = (head_dim + 31) / 32;
   if (key_hi < key_lo) return;
   const int page_last = key_hi / PAGE_TOKENS;
   for (int pi = page_first; pi <= page_last; pi += page_step) {
@@ -116,72 +192,8 @@ __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const 
     for (int half = 0; half < 2; ++half) {
       const int key0 = pi * PAGE_TOKENS + half * 32;
       if (key0 > key_hi || key0 + 31 < key_lo) continue;  // uniform over the wave
-      f32x4 sa[QT], sb[QT];
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt) {
-        sa[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
-        sb[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-#pragma unroll
-      for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
-        if (c < nchunk) {
-          const int d = c * 32 + g * 8;
-          bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0}, kb = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (d < head_dim) {
-            ka = load_bf16x8(kp + (size_t)(half * 32 + r) * head_dim + d);
-            kb = load_bf16x8(kp + (size_t)(half * 32 + 16 + r) * head_dim + d);
-          }
-#pragma unroll
-          for (int qt = 0; qt < QT; ++qt) {
-            sa[qt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qreg[qt][c], sa[qt], 0, 0, 0);
-            sb[qt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qreg[qt][c], sb[qt], 0, 0, 0);
-          }
-        }
-      }
-      bf16x8 pmat[QT];
-#pragma unroll
-      for (int qt = 0; qt < QT; ++qt) {
-        float mx = -INFINITY;
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int ja = key0 + g * 4 + i;
-          const int jb = ja + 16;
-          sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale : -INFINITY;
-          sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale : -INFINITY;
-          mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
-        }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-        const float m_new = fmaxf(st.m[qt], mx);
-        const float alpha = __expf(st.m[qt] - m_new);
-        st.m[qt] = m_new;
-        float psum = 0.f;
-        float pa[4], pb[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          pa[i] = __expf(sa[qt][i] - m_new);
-          pb[i] = __expf(sb[qt][i] - m_new);
-          psum += pa[i] + pb[i];
-        }
-        st.l[qt] = st.l[qt] * alpha + psum;
-        pmat[qt] = bf16x8{(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3],
-                          (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
-#pragma unroll
-        for (int dt = 0; dt < MAXDT; ++dt)
-          if (dt < ndt) st.acc[qt][dt] *= alpha;
-      }
-#pragma unroll
-      for (int dt = 0; dt < MAXDT; ++dt) {
-        if (dt < ndt) {
-          const bf16* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + half * 32 + g * 4;
-          const bf16x4 va = load_bf16x4(vrow);
-          const bf16x4 vb = load_bf16x4(vrow + 16);
-          const bf16x8 v = {va[0], va[1], va[2], va[3], vb[0], vb[1], vb[2], vb[3]};
-#pragma unroll
-          for (int qt = 0; qt < QT; ++qt)
-            st.acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat[qt], st.acc[qt][dt], 0, 0, 0);
-        }
-      }
+      half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, kp + (size_t)half * 32 * head_dim, head_dim, vp + half * 32,
+                           PAGE_TOKENS, head_dim, scale);
     }
   }
 }
@@ -266,6 +278,139 @@ __global__ void __launch_bounds__(WAVES* WAVE)
   attn_wave_pages<MAXDT, QT>(st, qreg, qpos, qlo, key_lo, key_hi, key_lo / PAGE_TOKENS, 1, bt, k_cache, v_cache,
                              page_elems, kh, head_dim, scale);
 
+  const int ndt = head_dim / 16;
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    float l = st.l[qt];
+    l += __shfl_xor(l, 16, WAVE);
+    l += __shfl_xor(l, 32, WAVE);
+    const int t = t0 + qt * 16 + r;
+    if (t < t_end) {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      bf16* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+#pragma unroll
+      for (int dt = 0; dt < MAXDT; ++dt) {
+        if (dt < ndt) {
+          const f32x4 a = st.acc[qt][dt];
+          const bf16x4 o = {(bf16)(a[0] * inv), (bf16)(a[1] * inv), (bf16)(a[2] * inv), (bf16)(a[3] * inv)};
+          *reinterpret_cast<bf16x4*>(orow + dt * 16 + g * 4) = o;
+        }
+      }
+    }
+  }
+}
+
+// ==========================================================================
+// prefill through LDS.  A block of 4 waves stages one page of keys and values
+// at a time in LDS; its waves are `hb` query heads of one kv group (they share
+// the page) times 4/hb runs of 16*QT consecutive query tokens.  The next page
+// is fetched into registers while the current one is multiplied.
+// ==========================================================================
+#define LDS_PAD 8  // elements: rows 16 bytes apart from a multiple of the bank count
+
+template <int MAXDT, int QT>
+__global__ void __launch_bounds__(256)
+    attn_prefill_lds_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+                            const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                            const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
+                            int n_qblocks, const int* __restrict__ block_table, int table_stride,
+                            const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
+                            int kvheads, int head_dim, float scale, int window, int hb) {
+  constexpr int KS = MAXDT * 16 + LDS_PAD;    // LDS row stride of the key page [64][KS]
+  constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
+  constexpr int CH = MAXDT / 2;               // 16-byte chunks a thread moves per page and operand (at most)
+  __shared__ __attribute__((aligned(16))) bf16 ks[PAGE_TOKENS * KS];
+  __shared__ __attribute__((aligned(16))) bf16 vs[MAXDT * 16 * VS];
+
+  const int qb = n_qblocks - 1 - blockIdx.x;  // long blocks first: they end last
+  const int group = nheads / kvheads;
+  const int tiles = group / hb;
+  const int kh = blockIdx.y / tiles;
+  const int wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int h = kh * group + (blockIdx.y % tiles) * hb + wave % hb;
+  const int t_begin = qblock_start[qb];
+  const int t_end = t_begin + qblock_len[qb];
+  const int seq = seq_of_token[t_begin];
+  if (seq < 0) return;  // whole block: uniform
+  const int* bt = block_table + (size_t)seq * table_stride;
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  // this wave's queries
+  const int t0 = t_begin + (wave / hb) * QT * 16;
+  const bool has_work = t0 < t_end;
+  bf16x8 qreg[QT][(MAXDT + 1) / 2];
+  int qpos[QT], qlo[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int t = t0 + qt * 16 + r;
+    const bool valid = t < t_end;
+    load_query<MAXDT>(qreg[qt], valid ? q + (size_t)t * q_stride + (size_t)h * head_dim : nullptr, head_dim);
+    qpos[qt] = valid ? positions[t] : -1;
+    qlo[qt] = (valid && window > 0 && qpos[qt] - window + 1 > 0) ? qpos[qt] - window + 1 : 0;
+  }
+  int wave_hi = -1, wave_lo = 0;
+  if (has_work) {
+    const int t_last = (t0 + QT * 16 < t_end ? t0 + QT * 16 : t_end) - 1;
+    wave_hi = positions[t_last];
+    const int first = positions[t0];
+    wave_lo = (window > 0 && first - window + 1 > 0) ? first - window + 1 : 0;
+  }
+  // the block's keys: tokens of a block are consecutive positions of one sequence
+  const int blk_first = positions[t_begin];
+  const int blk_hi = positions[t_end - 1];
+  const int blk_lo = (window > 0 && blk_first - window + 1 > 0) ? blk_first - window + 1 : 0;
+  const int page_first = blk_lo / PAGE_TOKENS, page_last = blk_hi / PAGE_TOKENS;
+
+  // cooperative copy: chunk id -> (row, 16-byte column) of the page in global memory and in LDS
+  const int k_chunks = PAGE_TOKENS * head_dim / 8;  // per page; the value page has as many
+  const int k_cols = head_dim / 8;
+  bf16x8 kbuf[CH], vbuf[CH];
+  auto fetch = [&](int pi) {
+    const size_t phys = (size_t)bt[pi];
+    const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
+    const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int id = threadIdx.x + j * 256;
+      if (id < k_chunks) {
+        kbuf[j] = load_bf16x8(kp + (size_t)id * 8);  // the page is contiguous
+        vbuf[j] = load_bf16x8(vp + (size_t)id * 8);
+      }
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int j = 0; j < CH; ++j) {
+      const int id = threadIdx.x + j * 256;
+      if (id < k_chunks) {
+        *reinterpret_cast<bf16x8*>(ks + (id / k_cols) * KS + (id % k_cols) * 8) = kbuf[j];
+        *reinterpret_cast<bf16x8*>(vs + (id / 8) * VS + (id % 8) * 8) = vbuf[j];
+      }
+    }
+  };
+
+  WaveState<MAXDT, QT> st;
+  wave_state_init(st);
+  fetch(page_first);
+  for (int pi = page_first; pi <= page_last; ++pi) {
+    stash();
+    __syncthreads();
+    if (pi < page_last) fetch(pi + 1);  // in flight while this page is multiplied
+    if (has_work) {
+#pragma unroll 1
+      for (int half = 0; half < 2; ++half) {  // not unrolled: the operands of one half fill the registers
+        const int key0 = pi * PAGE_TOKENS + half * 32;
+        if (key0 > wave_hi || key0 + 31 < wave_lo) continue;  // uniform over the wave
+        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + half * 32 * KS, KS, vs + half * 32, VS, head_dim, scale);
+      }
+    }
+    __syncthreads();  // the page is overwritten next
+  }
+
+  if (!has_work) return;
   const int ndt = head_dim / 16;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
@@ -542,33 +687,71 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
   return 0;
 }
 
+// How the bfloat16 prefill kernel cuts a step: the heads of a kv group that share a block, and the
+// query tokens a block covers.  Small head sizes go through LDS (4 waves = hb heads x 4/hb runs of
+// 16*QT tokens; QT = 4, or 2 when that is needed to give every compute unit two blocks); head
+// sizes above 128 keep the direct kernel (128 tokens).
+static void prefill_shape(int nheads, int kvheads, int head_dim, int n_tokens, int* hb, int* qt, int* qblock) {
+  const int group = nheads / kvheads;
+  if (head_dim > 128) {
+    *hb = 1, *qt = 0, *qblock = PREFILL_QBLOCK;
+    return;
+  }
+  *hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  const long blocks4 = (long)ceil_div(n_tokens, 64 * (4 / *hb)) * kvheads * (group / *hb);
+  *qt = (blocks4 >= 512 && head_dim <= 64) ? 4 : 2;  // 64 tokens per wave do not fit the registers at larger heads
+  *qblock = (4 / *hb) * *qt * 16;
+}
+
+extern "C" int fmsamd_attn_prefill_qblock(int nheads, int kvheads, int head_dim, int n_tokens) {
+  int hb, qt, qblock;
+  if (nheads <= 0 || kvheads <= 0 || nheads % kvheads) return PREFILL_QBLOCK;
+  prefill_shape(nheads, kvheads, head_dim, n_tokens, &hb, &qt, &qblock);
+  return qblock;
+}
+
 extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_stride,
                                         const int* positions, const int* seq_of_token, const int* qblock_start,
-                                        const int* qblock_len, int n_qblocks, const int* block_table, int table_stride,
-                                        const void* k_cache, const void* v_cache, int n_tokens, int nheads,
-                                        int kvheads, int head_dim, float scale, int window, hipStream_t stream) {
+                                        const int* qblock_len, int n_qblocks, int qblock_tokens,
+                                        const int* block_table, int table_stride, const void* k_cache,
+                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
+                                        float scale, int window, hipStream_t stream) {
   if (n_tokens == 0 || n_qblocks == 0) return 0;
   if (check_common("attn_prefill_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_prefill_bf16: head size %d is no multiple of 16", head_dim);
   FMS_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0, "attn_prefill_bf16: row strides must keep 16-byte alignment");
   FMS_REQUIRE(nheads <= 65535, "attn_prefill_bf16: too many heads");
-  dim3 grid(n_qblocks, nheads);
-#define FMS_PF(M, QT, WAVES)                                                                                        \
-  attn_prefill_bf16_kernel<M, QT, WAVES><<<grid, dim3(WAVES * WAVE), 0, stream>>>(                                  \
-      (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,          \
-      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window)
-  if (head_dim <= 64)
-    FMS_PF(4, 2, 4);
-  else if (head_dim <= 128)
-    FMS_PF(8, 2, 4);
-  else
-    FMS_PF(16, 1, 8);
-#undef FMS_PF
+  const int group = nheads / kvheads;
+  if (head_dim > 128) {
+    FMS_REQUIRE(qblock_tokens == PREFILL_QBLOCK, "attn_prefill_bf16: query blocks of %d tokens, %d expected",
+                qblock_tokens, PREFILL_QBLOCK);
+    dim3 grid(n_qblocks, nheads);
+    attn_prefill_bf16_kernel<16, 1, 8><<<grid, dim3(8 * WAVE), 0, stream>>>(
+        (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,
+        block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window);
+    FMS_LAUNCH_CHECK("attn_prefill_bf16");
+    return 0;
+  }
+  const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  const int qt = qblock_tokens * hb / 64;
+  FMS_REQUIRE((qt == 2 || qt == 4) && qt * 64 == qblock_tokens * hb,
+              "attn_prefill_bf16: query blocks of %d tokens do not fit %d heads per block", qblock_tokens, hb);
+  dim3 grid(n_qblocks, kvheads * (group / hb));
+#define FMS_PL(M, QT)                                                                                              \
+  attn_prefill_lds_kernel<M, QT><<<grid, dim3(256), 0, stream>>>(                                                  \
+      (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,         \
+      n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
+      scale, window, hb)
+  if (head_dim <= 64) {
+    if (qt == 2) FMS_PL(4, 2); else FMS_PL(4, 4);
+  } else {
+    FMS_REQUIRE(qt == 2, "attn_prefill_bf16: head size %d takes query blocks of %d tokens", head_dim, (4 / hb) * 32);
+    FMS_PL(8, 2);
+  }
+#undef FMS_PL
   FMS_LAUNCH_CHECK("attn_prefill_bf16");
   return 0;
 }
-
-extern "C" int fmsamd_attn_prefill_qblock() { return PREFILL_QBLOCK; }
 
 extern "C" long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits) {
   if (n_splits <= 1) return 0;

@@ -61,11 +61,12 @@ int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride
                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, float scale,
                         int window, hipStream_t stream);
 
-// bfloat16 prefill: query blocks of at most fmsamd_attn_prefill_qblock() consecutive tokens of one sequence
-int fmsamd_attn_prefill_qblock();
+// bfloat16 prefill: the step is cut into query blocks of at most fmsamd_attn_prefill_qblock(...) consecutive
+// tokens of one sequence; the same number goes into the call as qblock_tokens
+int fmsamd_attn_prefill_qblock(int nheads, int kvheads, int head_dim, int n_tokens);
 int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_stride, const int* positions,
                              const int* seq_of_token, const int* qblock_start, const int* qblock_len, int n_qblocks,
-                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
+                             int qblock_tokens, const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                              hipStream_t stream);
 

@@ -27,8 +27,8 @@ class StepBatch:
     slot_ids: torch.Tensor  # int32 [B], row of each sequence in the state tensors
     seq_starts: torch.Tensor  # int32 [B + 1], offsets of the sequences in the token arrays
     block_tables: Dict[int, torch.Tensor]  # group index -> int32 [B, pages]
-    qblock_start: Optional[torch.Tensor] = None  # query blocks of the bfloat16 prefill kernel
-    qblock_len: Optional[torch.Tensor] = None
+    # query blocks for the prefill attention kernel: block size -> (first token, length) of each block
+    qblocks: Dict[int, tuple] = dataclasses.field(default_factory=dict)
     logit_rows: Optional[torch.Tensor] = None  # int32 [n_wanted] token indices whose logits are wanted
     n_logit_rows: int = 0
 
@@ -40,9 +40,10 @@ def build_batch(
     starts: Sequence[int],
     want: Sequence[Sequence[int]],
     device,
-    qblock: int,
+    qblock_sizes: Sequence[int] = (),
 ) -> StepBatch:
-    """Index arrays of a step.  `starts[b]` is what cache.extend(slot, len(tokens[b])) returned."""
+    """Index arrays of a step.  `starts[b]` is what cache.extend(slot, len(tokens[b])) returned.
+    qblock_sizes: the block sizes in which mixers want the step's tokens cut (blocks never span sequences)."""
     B = len(slots)
     q_lens = [len(t) for t in tokens]
     T = sum(q_lens)
@@ -51,8 +52,9 @@ def build_batch(
     seq_of_token: List[int] = []
     seq_starts = [0]
     rows: List[int] = []
-    qb_start: List[int] = []
-    qb_len: List[int] = []
+    sizes = sorted(set(int(s) for s in qblock_sizes if s))
+    qb_start: Dict[int, List[int]] = {s: [] for s in sizes}
+    qb_len: Dict[int, List[int]] = {s: [] for s in sizes}
     for b in range(B):
         base = seq_starts[-1]
         flat_ids.extend(int(x) for x in tokens[b])
@@ -63,20 +65,23 @@ def build_batch(
             if not 0 <= w < q_lens[b]:
                 raise IndexError(f"wanted place {w} is outside the {q_lens[b]} tokens of sequence {b}")
             rows.append(base + w)
-        for off in range(0, q_lens[b], qblock):
-            qb_start.append(base + off)
-            qb_len.append(min(qblock, q_lens[b] - off))
+        for size in sizes:
+            for off in range(0, q_lens[b], size):
+                qb_start[size].append(base + off)
+                qb_len[size].append(min(size, q_lens[b] - off))
     tables = {g: cache.block_table(g, slots) for g in range(len(cache.groups))}
 
     # one host buffer, one copy
-    parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows, qb_start, qb_len]
-    sizes = [len(p) for p in parts]
+    parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows]
+    for size in sizes:
+        parts += [qb_start[size], qb_len[size]]
+    lengths = [len(p) for p in parts]
     table_sizes = {g: t.numel() for g, t in tables.items()}
-    total = sum(sizes) + sum(table_sizes.values())
+    total = sum(lengths) + sum(table_sizes.values())
     host = torch.empty(total, dtype=torch.int32, pin_memory=torch.cuda.is_available())
     off = 0
     spans = []
-    for p, n in zip(parts, sizes):
+    for p, n in zip(parts, lengths):
         if n:
             host[off : off + n] = torch.tensor(p, dtype=torch.int32)
         spans.append((off, n))
@@ -106,8 +111,7 @@ def build_batch(
         slot_ids=span(3),
         seq_starts=span(4),
         block_tables={g: dev[o : o + shape[0] * shape[1]].view(shape) for g, (o, shape) in table_spans.items()},
-        qblock_start=span(6),
-        qblock_len=span(7),
+        qblocks={size: (span(6 + 2 * i), span(7 + 2 * i)) for i, size in enumerate(sizes)},
         logit_rows=span(5),
         n_logit_rows=len(rows),
     )

@@ -55,8 +55,8 @@ class DecodeGraph:
         self.batch = StepBatch(
             n_tokens=rows, n_seqs=rows, slots=[], q_lens=[1] * rows, starts=[0] * rows, is_decode=True,
             max_context=max_context, token_ids=self.tokens, positions=self.positions, seq_of_token=self.seq_of_token,
-            slot_ids=self.slot_ids, seq_starts=self.seq_starts, block_tables=self.tables, qblock_start=None,
-            qblock_len=None, logit_rows=self.logit_rows, n_logit_rows=rows,
+            slot_ids=self.slot_ids, seq_starts=self.seq_starts, block_tables=self.tables,
+            logit_rows=self.logit_rows, n_logit_rows=rows,
         )
         # what the static buffers currently describe
         self.slots: Tuple[int, ...] = ()

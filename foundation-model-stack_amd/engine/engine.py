@@ -39,7 +39,6 @@ class Engine:
         if max_slots is None:
             max_slots = max(1, pages_for(max_tokens))
         self.cache = model.make_cache(max_tokens, max_slots)
-        self.qblock = ops.prefill_qblock()
         self.vocab = model.spec.vocab
         if use_graphs is None:
             use_graphs = not os.environ.get("FMS_AMD_NO_GRAPHS")
@@ -145,4 +144,11 @@ class Engine:
             if self.cache.length(s) + len(t) > self.cache.max_seq_len:
                 raise IndexError(f"sequence in slot {s} would reach {self.cache.length(s) + len(t)} tokens; the model has {self.cache.max_seq_len} positions")
         starts = [self.cache.extend(s, len(t)) for s, t in zip(slots, tokens)]
-        return build_batch(self.cache, slots, tokens, starts, want, self.device, self.qblock)
+        n_tokens = sum(len(t) for t in tokens)
+        sizes = set()
+        if any(len(t) > 1 for t in tokens):
+            for block in self.model.layers:
+                size = block.mixer.prefill_qblock(n_tokens, self.model.dtype)
+                if size:
+                    sizes.add(size)
+        return build_batch(self.cache, slots, tokens, starts, want, self.device, sizes)

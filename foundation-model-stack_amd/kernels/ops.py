@@ -293,6 +293,7 @@ def attention(
     max_context: int = 0,
     qblock_start: Optional[torch.Tensor] = None,
     qblock_len: Optional[torch.Tensor] = None,
+    qblock_tokens: int = 0,
     pages_per_block: int = 0,
     waves: int = 0,
     force_generic: bool = False,
@@ -341,7 +342,7 @@ def attention(
     _need_i32("qblock_len", qblock_len)
     check(lib.fmsamd_attn_prefill_bf16(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), positions.data_ptr(),
                                        seq_of_token.data_ptr(), qblock_start.data_ptr(), qblock_len.data_ptr(),
-                                       qblock_start.numel(), block_table.data_ptr(), block_table.stride(0),
+                                       qblock_start.numel(), int(qblock_tokens), block_table.data_ptr(), block_table.stride(0),
                                        k_cache.data_ptr(), v_cache.data_ptr(), *common_tail))
     return out
 
@@ -349,16 +350,20 @@ def attention(
 def decode_split(rows: int, n_pages: int):
     """(pages per split, waves per block) of the decode attention kernel.
 
-    rows = tokens x kv heads.  With 64 rows or more one block per row takes the whole context (its
-    waves share the pages and merge in LDS, no second kernel); fewer rows split the context over
-    several blocks so that the GPU still has some hundred waves to keep the cache in flight."""
-    waves = max(1, min(8, n_pages))
-    splits = 1 if rows >= 64 else min(-(-64 // max(rows, 1)), -(-n_pages // waves))
-    return max(1, -(-n_pages // splits)), waves
+    rows = tokens x kv heads.  A compute unit pulls only a small share of the memory bandwidth, so
+    the cache has to be spread over all of them: the context is cut into as many splits as give a
+    few hundred blocks; the waves of a block share its pages and merge in LDS, blocks of a row
+    merge in a second kernel.  With many rows one block takes the whole context."""
+    splits = max(1, min(-(-256 // max(rows, 1)), n_pages))
+    pages = -(-n_pages // splits)
+    waves = max(1, min(8 if splits > 1 else 4, pages))
+    return pages, waves
 
 
-def prefill_qblock() -> int:
-    return load().fmsamd_attn_prefill_qblock()
+def prefill_qblock(nheads: int, kvheads: int, head_dim: int, n_tokens: int) -> int:
+    """The number of consecutive query tokens of one sequence that a block of the bfloat16 prefill
+    kernel takes, for a step of n_tokens tokens; the step's query blocks are built with it."""
+    return load().fmsamd_attn_prefill_qblock(nheads, kvheads, head_dim, n_tokens)
 
 
 # --------------------------------------------------------------------------

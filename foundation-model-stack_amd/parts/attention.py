@@ -65,6 +65,11 @@ class MultiHeadAttention(Mixer):
         if self.position_encoder is not None:
             self.position_encoder.check_positions(max_position)
 
+    def prefill_qblock(self, n_tokens: int, dtype) -> int:
+        if dtype != torch.bfloat16 or self.head_dim % 16:
+            return 0  # the generic kernel takes tokens one by one
+        return ops.prefill_qblock(self.nheads, self.kvheads, self.head_dim, n_tokens)
+
     def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
         H, K, D = self.nheads, self.kvheads, self.head_dim
         table = batch.block_tables[cache.group]
@@ -85,10 +90,12 @@ class MultiHeadAttention(Mixer):
             if tables is None and self.position_encoder is not None:
                 self.position_encoder.adjust_qk(qkv, batch, H, K, D)
             ops.rope_kv_write(qkv, batch.positions, batch.seq_of_token, table, cos, sin, rot, keys, values, H, K, D)
+        size = 0 if batch.is_decode else self.prefill_qblock(batch.n_tokens, x.dtype)
+        qb_start, qb_len = batch.qblocks.get(size, (None, None))
         mixed = ops.attention(
             qkv, batch.positions, batch.seq_of_token, table, cache.keys, cache.values, H, K, D, self.scale, self.window,
             decode=batch.is_decode, max_context=batch.max_context,
-            qblock_start=batch.qblock_start, qblock_len=batch.qblock_len,
+            qblock_start=qb_start, qblock_len=qb_len, qblock_tokens=size,
         )
         return self.dense.forward(mixed)
 

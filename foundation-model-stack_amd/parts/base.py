@@ -76,6 +76,11 @@ class Mixer(Part):
     def check_step(self, max_position: int) -> None:
         """Raise if a token at `max_position` cannot be processed (for instance beyond a position table)."""
 
+    def prefill_qblock(self, n_tokens: int, dtype) -> int:
+        """If the mixer wants the tokens of a multi-token step cut into blocks (that never span two
+        sequences), the block size; the step's batch then carries them in `qblocks[size]`.  0: no."""
+        return 0
+
     def forward(self, x: torch.Tensor, batch, cache) -> torch.Tensor:
         raise NotImplementedError
 

@@ -260,7 +260,7 @@ def attention_case(ops, dtype, H, K, D, starts, lens, window=0, decode=False, sc
     wide[:, : H * D] = q_flat
     positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int()
     seq = torch.cat([torch.full((n,), b) for b, n in enumerate(lens)]).int()
-    qblock = ops.prefill_qblock()
+    qblock = kw.pop("qblock", None) or ops.prefill_qblock(H, K, D, T)
     qb_start, qb_len, base = [], [], 0
     for n in lens:
         for off in range(0, n, qblock):
@@ -271,7 +271,7 @@ def attention_case(ops, dtype, H, K, D, starts, lens, window=0, decode=False, sc
     out = ops.attention(
         dev(wide), dev(positions), dev(seq), dev(table), dev(kc), dev(vc), H, K, D, sc, window,
         decode=decode, max_context=max(totals),
-        qblock_start=dev(torch.tensor(qb_start, dtype=torch.int32)), qblock_len=dev(torch.tensor(qb_len, dtype=torch.int32)), **kw,
+        qblock_start=dev(torch.tensor(qb_start, dtype=torch.int32)), qblock_len=dev(torch.tensor(qb_len, dtype=torch.int32)), qblock_tokens=qblock, **kw,
     )
     want = reference_attention(qs, ks, vs, starts, H, K, scale=sc, window=window)
     torch.testing.assert_close(out.cpu().float(), want, **(dict(atol=3e-5, rtol=3e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)))
@@ -283,11 +283,17 @@ def test_attention_generic_f32(ops, H, K, D):
     attention_case(ops, torch.float32, H, K, D, starts=[299, 64], lens=[1, 1], decode=True)
 
 
-@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (6, 3, 128), (2, 2, 64), (32, 1, 32), (2, 1, 256), (5, 5, 80)])
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (6, 3, 128), (2, 2, 64), (32, 1, 32), (2, 1, 256), (5, 5, 80), (8, 2, 128), (12, 2, 64)])
 def test_attention_prefill_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 0, 0], lens=[200, 1, 33])
     # a chunk that continues a cached prefix
     attention_case(ops, torch.bfloat16, H, K, D, starts=[100, 64, 0], lens=[70, 5, 129])
+    if D <= 128:
+        # both shapes of a block: 16*2 and 16*4 tokens per wave
+        group = H // K
+        hb = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
+        for qt in ((2, 4) if D <= 64 else (2,)):
+            attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 30], lens=[300, 100], qblock=(4 // hb) * qt * 16)
 
 
 @pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (8, 2, 128), (2, 2, 64), (40, 2, 32), (2, 1, 256), (5, 5, 80)])

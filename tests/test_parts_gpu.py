@@ -129,13 +129,13 @@ def test_attention_part_prefill_then_decode(lib, dtype, H, K, D):
     view = LayerCache(group, keys, values, True, {})
     # prompts in one step
     starts = [cache.extend(s, n) for s, n in zip(slots, lens)]
-    batch = build_batch(cache, slots, [[0] * n for n in lens], starts, [[] for _ in lens], DEV, ops.prefill_qblock())
+    batch = build_batch(cache, slots, [[0] * n for n in lens], starts, [[] for _ in lens], DEV, [attn.prefill_qblock(sum(lens), dtype)])
     out = attn.forward(torch.cat([x[:n] for x, n in zip(xs, lens)]).to(DEV), batch, view).cpu().float()
     close(out, torch.cat([wt[:n] for wt, n in zip(want, lens)]), dtype)
     # three more tokens each, one at a time
     for i in range(3):
         starts = [cache.extend(s, 1) for s in slots]
-        batch = build_batch(cache, slots, [[0], [0]], starts, [[], []], DEV, ops.prefill_qblock())
+        batch = build_batch(cache, slots, [[0], [0]], starts, [[], []], DEV)
         out = attn.forward(torch.stack([x[n + i] for x, n in zip(xs, lens)]).to(DEV), batch, view).cpu().float()
         close(out, torch.stack([wt[n + i] for wt, n in zip(want, lens)]), dtype)
 
