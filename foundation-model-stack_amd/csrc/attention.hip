@@ -309,7 +309,7 @@ __global__ void __launch_bounds__(WAVES* WAVE)
 #define LDS_PAD 8  // elements: rows 16 bytes apart from a multiple of the bank count
 
 template <int MAXDT, int QT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
     attn_prefill_lds_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
