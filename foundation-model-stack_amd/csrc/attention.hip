@@ -80,6 +80,8 @@ __global__ void __launch_bounds__(GEN_THREADS)
   if (threadIdx.x < head_dim) o[threadIdx.x] = from_f32<T>(l_run > 0.f ? acc / l_run : 0.f);
 }
 
+#define LOG2E 1.4426950408889634f
+
 // ==========================================================================
 // MFMA core.  One wave owns 16*QT query columns and walks over pages of keys.
 // ==========================================================================
@@ -98,10 +100,14 @@ __device__ __forceinline__ bf16x4 load_bf16x4(const bf16* p) { return *reinterpr
 // qpos/qlo: visible keys of this lane's column are qlo <= key <= qpos (qpos < 0: no key).
 // kbase: key row 0 of the 32 keys, rows k_stride elements apart; vbase: column 0 of the 32 keys in the
 // transposed values, rows (head_dim of them) v_stride elements apart.  Global memory or LDS.
+// scale2 = softmax scale * log2(e): scores and running maxima live in the base-2 domain (exp2 is the
+// hardware's native exponential).  `full`: every one of the 32 keys is visible to every column of the
+// wave, so no mask is applied (true for all but the steps at the causal edge or a window's edge).
 template <int MAXDT, int QT>
 __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
                                           const int (&qpos)[QT], const int (&qlo)[QT], int key0, const bf16* kbase,
-                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, float scale) {
+                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, float scale2,
+                                          bool full) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
@@ -133,33 +139,45 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     float mx = -INFINITY;
+    if (full) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int ja = key0 + g * 4 + i;
-      const int jb = ja + 16;
-      sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale : -INFINITY;
-      sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale : -INFINITY;
-      mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
+      for (int i = 0; i < 4; ++i) {
+        sa[qt][i] *= scale2;
+        sb[qt][i] *= scale2;
+        mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ja = key0 + g * 4 + i;
+        const int jb = ja + 16;
+        sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale2 : -INFINITY;
+        sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale2 : -INFINITY;
+        mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
+      }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(st.m[qt], mx);
-    const float alpha = __expf(st.m[qt] - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(st.m[qt] - m_new);
     st.m[qt] = m_new;
     float psum = 0.f;
     float pa[4], pb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      pa[i] = __expf(sa[qt][i] - m_new);
-      pb[i] = __expf(sb[qt][i] - m_new);
+      pa[i] = __builtin_amdgcn_exp2f(sa[qt][i] - m_new);
+      pb[i] = __builtin_amdgcn_exp2f(sb[qt][i] - m_new);
       psum += pa[i] + pb[i];
     }
     st.l[qt] = st.l[qt] * alpha + psum;
     pmat[qt] = bf16x8{(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3],
                       (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
+    // the running maximum seldom moves after the first keys: rescale only when some column's did
+    if (__any(alpha != 1.f)) {
 #pragma unroll
-    for (int dt = 0; dt < MAXDT; ++dt)
-      if (dt < ndt) st.acc[qt][dt] *= alpha;
+      for (int dt = 0; dt < MAXDT; ++dt)
+        if (dt < ndt) st.acc[qt][dt] *= alpha;
+    }
   }
 #pragma unroll
   for (int dt = 0; dt < MAXDT; ++dt) {
@@ -181,7 +199,9 @@ __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const 
                                                 const int (&qpos)[QT], const int (&qlo)[QT], int key_lo, int key_hi,
                                                 int page_first, int page_step, const int* __restrict__ bt,
                                                 const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
-                                                size_t page_elems, int kh, int head_dim, float scale) {
+                                                size_t page_elems, int kh, int head_dim, float scale, int full_lo,
+                                                int full_hi) {
+  // full_lo..full_hi: the keys that every column of the wave sees (no mask needed inside)
   if (key_hi < key_lo) return;
   const int page_last = key_hi / PAGE_TOKENS;
   for (int pi = page_first; pi <= page_last; pi += page_step) {
@@ -193,7 +213,7 @@ __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const 
       const int key0 = pi * PAGE_TOKENS + half * 32;
       if (key0 > key_hi || key0 + 31 < key_lo) continue;  // uniform over the wave
       half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, kp + (size_t)half * 32 * head_dim, head_dim, vp + half * 32,
-                           PAGE_TOKENS, head_dim, scale);
+                           PAGE_TOKENS, head_dim, scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
     }
   }
 }
@@ -275,8 +295,11 @@ __global__ void __launch_bounds__(WAVES* WAVE)
 
   WaveState<MAXDT, QT> st;
   wave_state_init(st);
+  // every column sees the keys from the last token's window start up to the first token's position
+  const int full_hi = positions[t0];
+  const int full_lo = (window > 0 && key_hi - window + 1 > 0) ? key_hi - window + 1 : 0;
   attn_wave_pages<MAXDT, QT>(st, qreg, qpos, qlo, key_lo, key_hi, key_lo / PAGE_TOKENS, 1, bt, k_cache, v_cache,
-                             page_elems, kh, head_dim, scale);
+                             page_elems, kh, head_dim, scale, full_lo, full_hi);
 
   const int ndt = head_dim / 16;
 #pragma unroll
@@ -322,7 +345,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   __shared__ __attribute__((aligned(16))) bf16 ks[PAGE_TOKENS * KS];
   __shared__ __attribute__((aligned(16))) bf16 vs[MAXDT * 16 * VS];
 
-  const int qb = n_qblocks - 1 - blockIdx.x;  // long blocks first: they end last
+  // Blocks of a causal step differ in length.  Workgroups are handed to compute units in linear order, a
+  // full round at a time, so the rounds alternate between long-first and short-first: a unit that got a
+  // long block in one round gets a short one in the next.
+  const unsigned linear = blockIdx.x + blockIdx.y * gridDim.x;
+  const int qb = ((linear / 256) & 1) ? (int)blockIdx.x : n_qblocks - 1 - (int)blockIdx.x;
   const int group = nheads / kvheads;
   const int tiles = group / hb;
   const int kh = blockIdx.y / tiles;
@@ -351,12 +378,13 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     qpos[qt] = valid ? positions[t] : -1;
     qlo[qt] = (valid && window > 0 && qpos[qt] - window + 1 > 0) ? qpos[qt] - window + 1 : 0;
   }
-  int wave_hi = -1, wave_lo = 0;
+  int wave_hi = -1, wave_lo = 0, full_hi = -1, full_lo = 0;  // keys some / every column of the wave sees
   if (has_work) {
     const int t_last = (t0 + QT * 16 < t_end ? t0 + QT * 16 : t_end) - 1;
     wave_hi = positions[t_last];
-    const int first = positions[t0];
-    wave_lo = (window > 0 && first - window + 1 > 0) ? first - window + 1 : 0;
+    full_hi = positions[t0];
+    wave_lo = (window > 0 && full_hi - window + 1 > 0) ? full_hi - window + 1 : 0;
+    full_lo = (window > 0 && wave_hi - window + 1 > 0) ? wave_hi - window + 1 : 0;
   }
   // the block's keys: tokens of a block are consecutive positions of one sequence
   const int blk_first = positions[t_begin];
@@ -404,7 +432,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
       for (int half = 0; half < 2; ++half) {  // not unrolled: the operands of one half fill the registers
         const int key0 = pi * PAGE_TOKENS + half * 32;
         if (key0 > wave_hi || key0 + 31 < wave_lo) continue;  // uniform over the wave
-        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + half * 32 * KS, KS, vs + half * 32, VS, head_dim, scale);
+        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + half * 32 * KS, KS, vs + half * 32, VS, head_dim,
+                             scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
       }
     }
     __syncthreads();  // the page is overwritten next
@@ -444,7 +473,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 template <int MAXDT, int HALVES>
 __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
                                             int qlo, int key0, const bf16* __restrict__ kp,
-                                            const bf16* __restrict__ vp, int head_dim, float scale) {
+                                            const bf16* __restrict__ vp, int head_dim, float scale2) {
   // HALVES halves of 32 keys starting at key0 (kp/vp point at the page, `first` is the half inside it)
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
@@ -484,24 +513,33 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
       }
     }
     float mx = -INFINITY;
+    if (k0 + 31 <= qpos && k0 >= qlo) {  // uniform: all 32 keys are visible
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int ja = k0 + g * 4 + i;
-      const int jb = ja + 16;
-      sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] * scale : -INFINITY;
-      sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] * scale : -INFINITY;
-      mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
+      for (int i = 0; i < 4; ++i) {
+        sa[i] *= scale2;
+        sb[i] *= scale2;
+        mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ja = k0 + g * 4 + i;
+        const int jb = ja + 16;
+        sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] * scale2 : -INFINITY;
+        sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] * scale2 : -INFINITY;
+        mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
+      }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
     const float m_new = fmaxf(st.m[0], mx);
-    const float alpha = __expf(st.m[0] - m_new);
+    const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
     st.m[0] = m_new;
     float pa[4], pb[4], psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      pa[i] = __expf(sa[i] - m_new);
-      pb[i] = __expf(sb[i] - m_new);
+      pa[i] = __builtin_amdgcn_exp2f(sa[i] - m_new);
+      pb[i] = __builtin_amdgcn_exp2f(sb[i] - m_new);
       psum += pa[i] + pb[i];
     }
     st.l[0] = st.l[0] * alpha + psum;
@@ -573,10 +611,10 @@ __global__ void __launch_bounds__(MAXW* WAVE)
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
     if (MAXDT <= 8) {
-      decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale);
+      decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
     } else {  // large heads: half a page at a time keeps the loads in registers
-      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale);
-      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, scale);
+      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
+      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, scale * LOG2E);
     }
   }
 
@@ -607,7 +645,7 @@ __global__ void __launch_bounds__(MAXW* WAVE)
     float o = 0.f, lsum = 0.f;
     for (int w = 0; w < n_waves; ++w) {
       const float* src = lds + ((size_t)w * tile_cols + c) * cstride;
-      const float f = __expf(src[head_dim] - m);
+      const float f = __builtin_amdgcn_exp2f(src[head_dim] - m);  // maxima are base-2 logarithms
       o += f * src[d];
       lsum += f * src[head_dim + 1];
     }
@@ -643,7 +681,7 @@ __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
     float o = 0.f, l = 0.f;
     for (int s = first_split; s <= last_split; ++s) {
-      const float f = __expf(part_ml[(base + s) * 2] - m);
+      const float f = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m);  // maxima are base-2 logarithms
       o += f * part_o[(base + s) * head_dim + d];
       l += f * part_ml[(base + s) * 2 + 1];
     }
@@ -688,18 +726,18 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
 }
 
 // How the bfloat16 prefill kernel cuts a step: the heads of a kv group that share a block, and the
-// query tokens a block covers.  Small head sizes go through LDS (4 waves = hb heads x 4/hb runs of
-// 16*QT tokens; QT = 4, or 2 when that is needed to give every compute unit two blocks); head
-// sizes above 128 keep the direct kernel (128 tokens).
+// query tokens a block covers.  Head sizes up to 128 go through LDS (4 waves = hb heads x 4/hb runs of
+// 32 tokens); larger ones keep the direct kernel (128 tokens).
+#define LDS_QT 2
 static void prefill_shape(int nheads, int kvheads, int head_dim, int n_tokens, int* hb, int* qt, int* qblock) {
   const int group = nheads / kvheads;
+  (void)n_tokens;
   if (head_dim > 128) {
     *hb = 1, *qt = 0, *qblock = PREFILL_QBLOCK;
     return;
   }
   *hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-  const long blocks4 = (long)ceil_div(n_tokens, 64 * (4 / *hb)) * kvheads * (group / *hb);
-  *qt = (blocks4 >= 512 && head_dim <= 64) ? 4 : 2;  // 64 tokens per wave do not fit the registers at larger heads
+  *qt = LDS_QT;
   *qblock = (4 / *hb) * *qt * 16;
 }
 
@@ -733,21 +771,18 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     return 0;
   }
   const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-  const int qt = qblock_tokens * hb / 64;
-  FMS_REQUIRE((qt == 2 || qt == 4) && qt * 64 == qblock_tokens * hb,
-              "attn_prefill_bf16: query blocks of %d tokens do not fit %d heads per block", qblock_tokens, hb);
+  FMS_REQUIRE(qblock_tokens == (4 / hb) * LDS_QT * 16, "attn_prefill_bf16: query blocks of %d tokens, %d expected",
+              qblock_tokens, (4 / hb) * LDS_QT * 16);
   dim3 grid(n_qblocks, kvheads * (group / hb));
-#define FMS_PL(M, QT)                                                                                              \
-  attn_prefill_lds_kernel<M, QT><<<grid, dim3(256), 0, stream>>>(                                                  \
+#define FMS_PL(M)                                                                                                  \
+  attn_prefill_lds_kernel<M, LDS_QT><<<grid, dim3(256), 0, stream>>>(                                              \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,         \
       n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
       scale, window, hb)
-  if (head_dim <= 64) {
-    if (qt == 2) FMS_PL(4, 2); else FMS_PL(4, 4);
-  } else {
-    FMS_REQUIRE(qt == 2, "attn_prefill_bf16: head size %d takes query blocks of %d tokens", head_dim, (4 / hb) * 32);
-    FMS_PL(8, 2);
-  }
+  if (head_dim <= 64)
+    FMS_PL(4);
+  else
+    FMS_PL(8);
 #undef FMS_PL
   FMS_LAUNCH_CHECK("attn_prefill_bf16");
   return 0;

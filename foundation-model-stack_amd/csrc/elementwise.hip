@@ -260,21 +260,53 @@ __device__ __forceinline__ float activate(float x, int kind) {
   }
 }
 
-template <typename T, typename BiasT>
+// VEC elements per thread and step: 16 bytes of the activation type when the row length allows it
+template <int VEC, typename T, typename BiasT>
 __global__ void gated_act_kernel(const T* __restrict__ gu, const BiasT* __restrict__ bias, T* __restrict__ out,
                                  int hidden, int act) {
   const size_t t = blockIdx.y;
   const T* g = gu + t * 2 * hidden;
   const T* u = g + hidden;
   T* o = out + t * hidden;
-  for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < hidden; j += gridDim.x * blockDim.x) {
-    float gv = to_f32(g[j]), uv = to_f32(u[j]);
-    if (bias) {
-      gv += to_f32(bias[j]);
-      uv += to_f32(bias[hidden + j]);
+  for (int j = (blockIdx.x * blockDim.x + threadIdx.x) * VEC; j < hidden; j += gridDim.x * blockDim.x * VEC) {
+    __attribute__((aligned(16))) T gv[VEC], uv[VEC], ov[VEC];
+    if constexpr (VEC * sizeof(T) == 16) {
+      *reinterpret_cast<f32x4*>(gv) = *reinterpret_cast<const f32x4*>(g + j);
+      *reinterpret_cast<f32x4*>(uv) = *reinterpret_cast<const f32x4*>(u + j);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) gv[e] = g[j + e], uv[e] = u[j + e];
     }
-    o[j] = from_f32<T>(activate(gv, act) * uv);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      float a = to_f32(gv[e]), b = to_f32(uv[e]);
+      if (bias) {
+        a += to_f32(bias[j + e]);
+        b += to_f32(bias[hidden + j + e]);
+      }
+      ov[e] = from_f32<T>(activate(a, act) * b);
+    }
+    if constexpr (VEC * sizeof(T) == 16) {
+      *reinterpret_cast<f32x4*>(o + j) = *reinterpret_cast<const f32x4*>(ov);
+    } else {
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) o[j + e] = ov[e];
+    }
   }
+}
+
+template <typename T, typename BiasT>
+static void launch_gated_act(const void* gu, const void* bias, void* out, int n_tokens, int hidden, int act,
+                             hipStream_t stream) {
+  constexpr int VEC = 16 / sizeof(T);
+  const bool wide = hidden % VEC == 0 && (((size_t)gu | (size_t)out) & 15) == 0;
+  const int per_thread = wide ? VEC : 1;
+  const int blocks = ceil_div(hidden, 256 * per_thread);
+  dim3 grid(blocks > 64 ? 64 : blocks, n_tokens);
+  if (wide)
+    gated_act_kernel<VEC, T, BiasT><<<grid, 256, 0, stream>>>((const T*)gu, (const BiasT*)bias, (T*)out, hidden, act);
+  else
+    gated_act_kernel<1, T, BiasT><<<grid, 256, 0, stream>>>((const T*)gu, (const BiasT*)bias, (T*)out, hidden, act);
 }
 
 extern "C" int fmsamd_gated_act(const void* gu, const void* bias, int bias_dtype, void* out, int dtype, int n_tokens,
@@ -283,15 +315,14 @@ extern "C" int fmsamd_gated_act(const void* gu, const void* bias, int bias_dtype
   FMS_REQUIRE(n_tokens > 0 && hidden > 0, "gated_act: bad sizes T=%d hidden=%d", n_tokens, hidden);
   FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gated_act: unknown activation %d", act);
   FMS_REQUIRE(n_tokens <= 65535, "gated_act: %d tokens exceed one launch (65535)", n_tokens);
-  dim3 grid(ceil_div(hidden, 256) > 64 ? 64 : ceil_div(hidden, 256), n_tokens);
   if (dtype == FMS_F32 && (bias == nullptr || bias_dtype == FMS_F32))
-    gated_act_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)gu, (const float*)bias, (float*)out, hidden, act);
+    launch_gated_act<float, float>(gu, bias, out, n_tokens, hidden, act, stream);
   else if (dtype == FMS_BF16 && (bias == nullptr || bias_dtype == FMS_BF16))
-    gated_act_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)gu, (const bf16*)bias, (bf16*)out, hidden, act);
+    launch_gated_act<bf16, bf16>(gu, bias, out, n_tokens, hidden, act, stream);
   else if (dtype == FMS_BF16 && bias_dtype == FMS_F32)
-    gated_act_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)gu, (const float*)bias, (bf16*)out, hidden, act);
+    launch_gated_act<bf16, float>(gu, bias, out, n_tokens, hidden, act, stream);
   else if (dtype == FMS_F32 && bias_dtype == FMS_BF16)
-    gated_act_kernel<float, bf16><<<grid, 256, 0, stream>>>((const float*)gu, (const bf16*)bias, (float*)out, hidden, act);
+    launch_gated_act<float, bf16>(gu, bias, out, n_tokens, hidden, act, stream);
   else
     FMS_REQUIRE(false, "gated_act: unknown dtypes %d/%d", dtype, bias_dtype);
   FMS_LAUNCH_CHECK("gated_act");

@@ -288,12 +288,7 @@ def test_attention_prefill_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 0, 0], lens=[200, 1, 33])
     # a chunk that continues a cached prefix
     attention_case(ops, torch.bfloat16, H, K, D, starts=[100, 64, 0], lens=[70, 5, 129])
-    if D <= 128:
-        # both shapes of a block: 16*2 and 16*4 tokens per wave
-        group = H // K
-        hb = 4 if group % 4 == 0 else (2 if group % 2 == 0 else 1)
-        for qt in ((2, 4) if D <= 64 else (2,)):
-            attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 30], lens=[300, 100], qblock=(4 // hb) * qt * 16)
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 30], lens=[300, 100])
 
 
 @pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (8, 2, 128), (2, 2, 64), (40, 2, 32), (2, 1, 256), (5, 5, 80)])
