@@ -84,10 +84,28 @@ int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias,
                     int K, hipStream_t stream);
 int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const void* bias, int bias_dtype, void* c, int out_dtype,
                      long ldc, int M, int N, int K, hipStream_t stream);
+// A row norm left to the product that reads the rows: the rows hold stream * norm weight, and the sums of
+// squares of the stream come as `count` partial sums per row (partials[m * count + i]).  The product is
+// multiplied by rsqrt(sum / K + eps) of its row before the bias.  A null pointer (or null partials): none.
+typedef struct {
+  const float* partials;
+  int count;
+  float eps;
+} fmsamd_row_scale;
+
+// at most 64 rows: the weights stream once through MFMA registers
 int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
-                            int out_dtype, long ldo, int M, int N, int K, hipStream_t stream);
+                            int out_dtype, long ldo, int M, int N, int K, const fmsamd_row_scale* row_scale,
+                            hipStream_t stream);
 int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
-                                  int out_dtype, long ldo, int M, int hidden, int K, int act, hipStream_t stream);
+                                  int out_dtype, long ldo, int M, int hidden, int K, int act,
+                                  const fmsamd_row_scale* row_scale, hipStream_t stream);
+// resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, ceil(N/16)] = sums of
+// squares of resid by tiles of 16 columns.  At most 32 rows.
+int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
+                                     float* resid, long ldr, const void* norm_w, int norm_w_dtype, void* scaled,
+                                     long ldo, float* partials, int M, int N, int K,
+                                     const fmsamd_row_scale* row_scale, hipStream_t stream);
 
 // qkv = x W^T (+ bias) for at most 32 rows with the rotation and the cache write fused into the epilogue;
 // only the query columns of `out` are written
@@ -95,7 +113,7 @@ int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const vo
                                 long ldo, int M, int K, const int* positions, const int* seq_of_token,
                                 const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
                                 int rot_dim, int max_pos, void* k_cache, void* v_cache, int nheads, int kvheads,
-                                int head_dim, hipStream_t stream);
+                                int head_dim, const fmsamd_row_scale* row_scale, hipStream_t stream);
 
 // token choice; rng_state is [rows][2] uint64 (seed, counter), advanced by the kernel
 int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature, int top_k,

@@ -203,6 +203,26 @@ __device__ __forceinline__ float sk_activate(float x, int kind) {
 #define EPI_GATED 1  // the block's second tile is the "up" half: out = act(first) * second, N is the hidden size
 #define EPI_ROPE 2   // the output row is [queries | keys | values] of attention: rotate q and k, store q, and
                      // write k and v into their cache pages (layout: see rope.hip)
+#define EPI_RESID 3  // add the product to the float32 residual stream in place, store the new stream times the
+                     // next norm's weight in the activation type, and leave the rows' sums of squares by tile
+
+// The rows of x are not yet divided by their root mean square: the kernel that made them left, for each
+// row, `count` partial sums of squares (partials[m * count + i]).  The product is multiplied by
+// rsqrt(sum / width + eps) of its row before the bias.  partials == null: the rows are taken as they are.
+struct RowScale {
+  const float* partials;
+  int count;
+  float inv_width, eps;
+};
+
+struct ResidEpilogue {
+  float* resid;  // [M, N] float32, read and written
+  long ldr;
+  const void* norm_w;  // [N] or null
+  int norm_w_f32;
+  float* partials;  // [M, tiles]: sum over the tile's 16 columns of the new stream squared
+  int tiles;
+};
 
 struct RopeEpilogue {
   const int* positions;     // [M]
@@ -226,10 +246,11 @@ template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typena
 __global__ void __launch_bounds__(SK_WAVES* WAVE)
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
-                       RopeEpilogue rope) {
+                       RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
   constexpr bool GATED = EPI == EPI_GATED;
   __shared__ float red[SK_WAVES][NTB][MT][16][17];
   __shared__ int s_pos[MT * 16], s_seq[MT * 16], s_page[MT * 16];
+  __shared__ float s_scale[MT * 16];
   const int wave = threadIdx.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
@@ -245,6 +266,54 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       if (seq >= 0 && rope.k_cache) page = rope.block_table[(size_t)seq * rope.table_stride + pos / PAGE_TOKENS];
     }
     s_pos[m] = pos, s_seq[m] = seq, s_page[m] = page;
+  }
+
+  // Loads whose data the epilogue needs are issued here, ahead of the weight stream, so that their latency
+  // is not paid at the end: the first partial sums of a deferred row norm (a wave per row, four rows and
+  // 256 sums deep) and the residual stream with the next norm's weight.
+  constexpr int PRE_ROWS = 4, PRE_DEPTH = 4;
+  float pre[PRE_ROWS][PRE_DEPTH];
+  if (scale.partials != nullptr) {
+#pragma unroll
+    for (int i = 0; i < PRE_ROWS; ++i)
+#pragma unroll
+      for (int j = 0; j < PRE_DEPTH; ++j) {
+        const int m = wave + i * SK_WAVES, b = lane + j * WAVE;
+        pre[i][j] = (m < M && b < scale.count) ? scale.partials[(size_t)m * scale.count + b] : 0.f;
+      }
+  }
+  constexpr int OUT_TILES = GATED ? 1 : NTB;
+  constexpr int ROUNDS = (OUT_TILES * MT * 256 + SK_WAVES * WAVE - 1) / (SK_WAVES * WAVE);
+  float pre_resid[ROUNDS], pre_nw[ROUNDS];  // EPI_ROPE: cosine and sine of the element's angle
+  if (EPI == EPI_ROPE) {
+#pragma unroll
+    for (int rd = 0; rd < ROUNDS; ++rd) {
+      const int idx = threadIdx.x + rd * SK_WAVES * WAVE;
+      const int m = ((idx >> 8) % MT) * 16 + ((idx >> 4) & 15);
+      const int n = n0 + ((idx >> 8) / MT) * 16 + (idx & 15);
+      const int hh = n / rope.head_dim, d = n - hh * rope.head_dim;
+      pre_resid[rd] = 1.f, pre_nw[rd] = 0.f;
+      if (idx < OUT_TILES * MT * 256 && m < M && n < N && hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr &&
+          d < rope.rot_dim) {
+        const int pos = rope.positions[m];
+        const int tpos = pos < rope.max_pos ? pos : rope.max_pos - 1;  // the host has checked the range
+        pre_resid[rd] = rope.cos_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
+        pre_nw[rd] = rope.sin_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
+      }
+    }
+  }
+  if (EPI == EPI_RESID) {
+#pragma unroll
+    for (int rd = 0; rd < ROUNDS; ++rd) {
+      const int idx = threadIdx.x + rd * SK_WAVES * WAVE;
+      const int m = ((idx >> 8) % MT) * 16 + ((idx >> 4) & 15);
+      const int n = n0 + ((idx >> 8) / MT) * 16 + (idx & 15);
+      const bool live = idx < OUT_TILES * MT * 256 && m < M && n < N;
+      pre_resid[rd] = live ? res.resid[(size_t)m * res.ldr + n] : 0.f;
+      pre_nw[rd] = 1.f;
+      if (live && res.norm_w != nullptr)
+        pre_nw[rd] = res.norm_w_f32 ? ((const float*)res.norm_w)[n] : to_f32(((const bf16*)res.norm_w)[n]);
+    }
   }
 
   const bf16* wrow[NTB];
@@ -308,11 +377,35 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
     for (int j = 0; j < MT; ++j)
 #pragma unroll
       for (int e = 0; e < 4; ++e) red[wave][i][j][g * 4 + e][r] = acc[i][j][e];
+
+  if (scale.partials != nullptr) {
+    // the rows' scales: partial sums in a fixed order, the same bits whatever the launch looks like
+#pragma unroll
+    for (int i = 0; i < PRE_ROWS; ++i) {
+      const int m = wave + i * SK_WAVES;
+      if (m < M) {
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < PRE_DEPTH; ++j) sum += pre[i][j];
+        for (int b = lane + PRE_DEPTH * WAVE; b < scale.count; b += WAVE) sum += scale.partials[(size_t)m * scale.count + b];
+        sum = wave_sum(sum);
+        if (lane == 0) s_scale[m] = rsqrtf(sum * scale.inv_width + scale.eps);
+      }
+    }
+    for (int m = wave + PRE_ROWS * SK_WAVES; m < M; m += SK_WAVES) {
+      float sum = 0.f;
+      for (int b = lane; b < scale.count; b += WAVE) sum += scale.partials[(size_t)m * scale.count + b];
+      sum = wave_sum(sum);
+      if (lane == 0) s_scale[m] = rsqrtf(sum * scale.inv_width + scale.eps);
+    }
+  }
   __syncthreads();
 
-  constexpr int OUT_TILES = GATED ? 1 : NTB;
   // every thread of a wave runs the same number of rounds (the rotation reads its neighbour's value)
-  for (int idx = threadIdx.x; idx < OUT_TILES * MT * 256; idx += blockDim.x) {
+#pragma unroll
+  for (int rd = 0; rd < ROUNDS; ++rd) {
+    const int idx = threadIdx.x + rd * SK_WAVES * WAVE;
+    if (idx >= OUT_TILES * MT * 256) break;  // whole waves leave together: the tile count is a multiple of 64
     const int nn = idx & 15;           // n within tile: fastest, so that stores of a row are contiguous
     const int mm = (idx >> 4) & 15;    // m within tile
     const int tj = (idx >> 8) % MT;    // m tile
@@ -323,11 +416,14 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
     float v = 0.f;
 #pragma unroll
     for (int wv = 0; wv < SK_WAVES; ++wv) v += red[wv][ti][tj][nn][mm];
+    const float row_scale = (scale.partials != nullptr && m < M) ? s_scale[m] : 1.f;
+    v *= row_scale;
     if (EPI == EPI_GATED) {
       if (!live) continue;
       float u = 0.f;
 #pragma unroll
       for (int wv = 0; wv < SK_WAVES; ++wv) u += red[wv][1][tj][nn][mm];
+      u *= row_scale;
       if (bias) {
         v += to_f32(bias[n]);
         u += to_f32(bias[tile2_offset + n]);
@@ -340,10 +436,8 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       const int D = rope.head_dim;
       const int hh = n / D, d = n - hh * D;
       const int pos = s_pos[m], seq = s_seq[m];
-      if (hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr && d < rope.rot_dim) {
-        const int tpos = pos < rope.max_pos ? pos : rope.max_pos - 1;  // the host has checked the range
-        const float c = rope.cos_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
-        const float sn = rope.sin_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
+      {
+        const float c = pre_resid[rd], sn = pre_nw[rd];  // 1 and 0 where nothing rotates
         v = (d & 1) ? sn * partner + c * v : c * v - sn * partner;
       }
       if (hh < rope.nheads) {
@@ -359,6 +453,19 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
           rope.v_cache[(size_t)s_page[m] * page_elems + ((size_t)kh * D + d) * PAGE_TOKENS + in_page] = (bf16)v;
         }
       }
+    } else if (EPI == EPI_RESID) {
+      float stream = 0.f;
+      if (live) {
+        if (bias) v += to_f32(bias[n]);
+        stream = pre_resid[rd] + v;
+        res.resid[(size_t)m * res.ldr + n] = stream;
+        out[(size_t)m * ldo + n] = from_f32<OutT>(stream * pre_nw[rd]);
+      }
+      // the 16 columns of a tile sit in 16 neighbouring lanes
+      float sq = stream * stream;
+#pragma unroll
+      for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, WAVE);
+      if (nn == 0 && m < M && n0 + ti * 16 < N) res.partials[(size_t)m * res.tiles + blockIdx.x * NTB + ti] = sq;
     } else {
       if (!live) continue;
       if (bias) v += to_f32(bias[n]);
@@ -370,19 +477,20 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 template <int NTB, int MT, int EPI>
 static void launch_skinny(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                           int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int blocks,
-                          hipStream_t stream, RopeEpilogue rope = RopeEpilogue{}) {
+                          hipStream_t stream, RowScale scale, RopeEpilogue rope = RopeEpilogue{},
+                          ResidEpilogue res = ResidEpilogue{}) {
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
   constexpr int SK_WAVES = NTB * MT > 4 ? 4 : 8;
   constexpr int UNR = (NTB + MT) <= 2 ? 4 : ((NTB + MT) <= 4 ? 2 : 1);
 #define FMS_SK(O, B)                                                                                 \
   skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, EPI, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(     \
-      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, rope)
+      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, scale, rope, res)
   if (out_dtype == FMS_BF16) {
     if (fb)
       FMS_SK(bf16, float);
     else
       FMS_SK(bf16, bf16);
-  } else if (EPI != EPI_ROPE) {
+  } else if (EPI != EPI_ROPE && EPI != EPI_RESID) {
     if (fb)
       FMS_SK(float, float);
     else
@@ -391,10 +499,22 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
 #undef FMS_SK
 }
 
+// Checks a deferred row norm and turns it into the kernel's argument.
+static int row_scale_of(const fmsamd_row_scale* in, int K, RowScale* out) {
+  *out = RowScale{nullptr, 0, 0.f, 0.f};
+  if (in == nullptr || in->partials == nullptr) return 0;
+  FMS_REQUIRE(in->count > 0 && in->eps >= 0.f, "deferred row norm: %d partial sums, eps %g", in->count, (double)in->eps);
+  *out = RowScale{in->partials, in->count, 1.f / (float)K, in->eps};
+  return 0;
+}
+
 // out[M, N] = x[M, K] w[N, K]^T (+ bias).  M <= 64.
 extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
-                                       void* out, int out_dtype, long ldo, int M, int N, int K, hipStream_t stream) {
+                                       void* out, int out_dtype, long ldo, int M, int N, int K,
+                                       const fmsamd_row_scale* row_scale, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
+  RowScale scale;
+  if (row_scale_of(row_scale, K, &scale)) return -1;
   FMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_bf16: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N, "gemm_skinny_bf16: leading dimensions too small");
@@ -404,7 +524,7 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   const bool two = N >= 16384;
   const int blocks = ceil_div(N, two ? 32 : 16);
 #define FMS_LS(NTB, MT) \
-  launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, blocks, stream)
+  launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, blocks, stream, scale)
   if (two) {
     if (mt == 1) FMS_LS(2, 1); else if (mt == 2) FMS_LS(2, 2); else if (mt == 3) FMS_LS(2, 3); else FMS_LS(2, 4);
   } else {
@@ -418,8 +538,10 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
 // out[M, hidden] = act(x Wg^T + bg) * (x Wu^T + bu) with w = [Wg; Wu] stacked, [2*hidden, K].  M <= 64.
 extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias,
                                              int bias_dtype, void* out, int out_dtype, long ldo, int M, int hidden,
-                                             int K, int act, hipStream_t stream) {
+                                             int K, int act, const fmsamd_row_scale* row_scale, hipStream_t stream) {
   if (M == 0 || hidden == 0) return 0;
+  RowScale scale;
+  if (row_scale_of(row_scale, K, &scale)) return -1;
   FMS_REQUIRE(M > 0 && M <= 64 && hidden > 0 && K > 0, "gemm_skinny_gated_bf16: bad sizes M=%d hidden=%d K=%d (M <= 64)",
               M, hidden, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_gated_bf16: K=%d and the row stride %ld must be multiples of 8", K,
@@ -430,7 +552,8 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
   const int mt = ceil_div(M, 16);
   const int blocks = ceil_div(hidden, 16);
 #define FMS_LG(MT) \
-  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, blocks, stream)
+  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, blocks, \
+                                  stream, scale)
   if (mt == 1) FMS_LG(1); else if (mt == 2) FMS_LG(2); else if (mt == 3) FMS_LG(3); else FMS_LG(4);
 #undef FMS_LG
   FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
@@ -445,9 +568,11 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
                                            const int* seq_of_token, const int* block_table, int table_stride,
                                            const float* cos_t, const float* sin_t, int rot_dim, int max_pos,
                                            void* k_cache, void* v_cache, int nheads, int kvheads, int head_dim,
-                                           hipStream_t stream) {
+                                           const fmsamd_row_scale* row_scale, hipStream_t stream) {
   if (M == 0) return 0;
   const int N = (nheads + 2 * kvheads) * head_dim;
+  RowScale scale;
+  if (row_scale_of(row_scale, K, &scale)) return -1;
   FMS_REQUIRE(M > 0 && M <= 32 && K > 0 && nheads > 0 && kvheads > 0 && head_dim > 0,
               "qkv_rope_skinny_bf16: bad sizes M=%d K=%d (M <= 32)", M, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "qkv_rope_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
@@ -462,9 +587,44 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
                     max_pos, (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim};
   const int blocks = N / 16;
   if (M <= 16)
-    launch_skinny<1, 1, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, rope);
+    launch_skinny<1, 1, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
+                                  rope);
   else
-    launch_skinny<1, 2, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, rope);
+    launch_skinny<1, 2, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
+                                  rope);
   FMS_LAUNCH_CHECK("qkv_rope_skinny_bf16");
+  return 0;
+}
+
+// The last product of a residual branch, fused with what follows it in a pre-norm block:
+//   resid[M, N] += x w^T (+ bias)                      float32, in place
+//   scaled[M, N] = resid * norm_w                      bfloat16: the next norm's input, not yet divided by its
+//                                                      root mean square
+//   partials[m, i] = sum over columns 16 i .. 16 i + 15 of resid[m]^2      [M, ceil(N / 16)]
+// A product that takes `scaled` with these partials as its deferred row norm then equals the product of the
+// normed stream.  M <= 32.
+extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias,
+                                                int bias_dtype, float* resid, long ldr, const void* norm_w,
+                                                int norm_w_dtype, void* scaled, long ldo, float* partials, int M, int N,
+                                                int K, const fmsamd_row_scale* row_scale, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  FMS_REQUIRE(M > 0 && M <= 32 && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 32)", M, N, K);
+  FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_residual_bf16: K=%d and the row stride %ld must be multiples of 8",
+              K, ldx);
+  FMS_REQUIRE(ldx >= K && ldo >= N && ldr >= N, "gemm_skinny_residual_bf16: leading dimensions too small");
+  FMS_REQUIRE(norm_w == nullptr || norm_w_dtype == FMS_BF16 || norm_w_dtype == FMS_F32,
+              "gemm_skinny_residual_bf16: unknown norm weight dtype %d", norm_w_dtype);
+  FMS_REQUIRE(resid != nullptr && scaled != nullptr && partials != nullptr, "gemm_skinny_residual_bf16: null buffer");
+  RowScale scale;
+  if (row_scale_of(row_scale, K, &scale)) return -1;
+  const int blocks = ceil_div(N, 16);
+  ResidEpilogue res{resid, ldr, norm_w, norm_w_dtype == FMS_F32, partials, blocks};
+  if (M <= 16)
+    launch_skinny<1, 1, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
+                                   RopeEpilogue{}, res);
+  else
+    launch_skinny<1, 2, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
+                                   RopeEpilogue{}, res);
+  FMS_LAUNCH_CHECK("gemm_skinny_residual_bf16");
   return 0;
 }

@@ -81,6 +81,11 @@ class DecoderModel(Part):
             else:
                 group, keys, values = -1, None, None
             view = LayerCache(group, keys, values, entry.cache_of is None, cache.state_of_entry(n))
-            block.forward(stream, batch, view, self.dtype)
-        normed = self.final_norm.add_norm(stream.resid, stream.pending, self.dtype, rows=batch.logit_rows)
+            if getattr(block, "fuses_next_norm", False) and n + 1 < len(self.schedule):
+                # the norm that reads the stream next, so that this block's last product can prepare its input
+                first_norm = getattr(self.layers[self.schedule[n + 1].layer], "first_norm", None)
+                block.forward(stream, batch, view, self.dtype, next_norm=first_norm() if first_norm else None)
+            else:
+                block.forward(stream, batch, view, self.dtype)
+        normed = stream.normed(self.final_norm, self.dtype, rows=batch.logit_rows)
         return self.head.forward(normed)

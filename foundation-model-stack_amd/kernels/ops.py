@@ -9,6 +9,7 @@ the host what its kernel and grid assume before launching.
 
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Optional
 
@@ -184,6 +185,30 @@ def _check_batch_index(positions, seq_of_token, block_table, n_tokens: int) -> N
         raise ValueError("positions and seq_of_token must have an entry per token")
 
 
+class RowNorm:
+    """A row norm left to the product that reads the rows.  The rows hold stream * norm weight; `partials`
+    [M, count] float32 are partial sums of squares of the stream's rows; the product multiplies its result
+    by rsqrt(sum / K + eps) per row before the bias."""
+
+    def __init__(self, partials: torch.Tensor, eps: float):
+        if partials.dtype != torch.float32 or partials.dim() != 2 or not partials.is_contiguous():
+            raise ValueError("the partial sums of a deferred row norm are a contiguous float32 [M, count] tensor")
+        self.partials, self.eps = partials, float(eps)
+
+
+class _RowScaleArg(ctypes.Structure):
+    _fields_ = [("partials", ctypes.c_void_p), ("count", ctypes.c_int), ("eps", ctypes.c_float)]
+
+
+def _row_scale(row_norm: Optional[RowNorm], rows: int):
+    if row_norm is None:
+        return None
+    _need_cuda(row_norm.partials)
+    if row_norm.partials.shape[0] != rows:
+        raise ValueError(f"deferred row norm has {row_norm.partials.shape[0]} rows, the product {rows}")
+    return ctypes.byref(_RowScaleArg(row_norm.partials.data_ptr(), row_norm.partials.shape[1], row_norm.eps))
+
+
 def qkv_rope_write(
     x: torch.Tensor,
     weight: torch.Tensor,
@@ -199,6 +224,7 @@ def qkv_rope_write(
     nheads: int,
     kvheads: int,
     head_dim: int,
+    row_norm: Optional[RowNorm] = None,
 ) -> torch.Tensor:
     """The fused qkv projection of a decode step (at most 32 rows, bfloat16): x W^T (+ bias), q and k
     rotated, k and v written into their cache pages.  Returns the [M, (H+2K)*D] buffer whose query
@@ -229,7 +255,7 @@ def qkv_rope_write(
         x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
         out.data_ptr(), out.stride(0), M, K, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
         block_table.stride(0), _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, max_pos, _ptr(k_cache),
-        _ptr(v_cache), nheads, kvheads, head_dim, _stream()))
+        _ptr(v_cache), nheads, kvheads, head_dim, _row_scale(row_norm, M), _stream()))
     return out
 
 
@@ -380,6 +406,7 @@ def linear(
     bias: Optional[torch.Tensor] = None,
     out_dtype: Optional[torch.dtype] = None,
     allow_library: bool = True,
+    row_norm: Optional[RowNorm] = None,
 ) -> torch.Tensor:
     """x [M, K] @ weight[N, K]^T (+ bias) -> [M, N].
 
@@ -402,6 +429,8 @@ def linear(
         raise ValueError(f"bias must be a contiguous [{N}] tensor")
     out_dtype = out_dtype or x.dtype
     lib = load()
+    if row_norm is not None and not (weight.dtype == x.dtype == torch.bfloat16 and M <= SKINNY_FAST_ROWS):
+        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 32 rows")
     if weight.dtype == torch.float32:
         xf = x if x.dtype == torch.float32 else cast(x.contiguous(), torch.float32)
         bf = bias if bias is None or bias.dtype == torch.float32 else cast(bias, torch.float32)
@@ -421,7 +450,7 @@ def linear(
     if M <= SKINNY_FAST_ROWS or (M <= SKINNY_MAX_ROWS and not (allow_library and out_dtype == torch.bfloat16)):
         out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         check(lib.fmsamd_gemm_skinny_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), bcode, out.data_ptr(),
-                                          _code(out_dtype), out.stride(0), M, N, K, _stream()))
+                                          _code(out_dtype), out.stride(0), M, N, K, _row_scale(row_norm, M), _stream()))
         return out
     if allow_library and out_dtype == torch.bfloat16:
         out = torch.matmul(x, weight.t())  # vendor library GEMM, float32 accumulation
@@ -434,8 +463,47 @@ def linear(
     return out
 
 
+def linear_into_stream(
+    x: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    resid: torch.Tensor,
+    norm_weight: Optional[torch.Tensor],
+    eps: float,
+    row_norm: Optional[RowNorm] = None,
+):
+    """The last product of a residual branch with what follows it (bfloat16, at most 32 rows):
+    resid += x W^T (+ bias) in float32 in place.  Returns (scaled, RowNorm): scaled = resid * norm_weight in
+    bfloat16 and the sums of squares of resid's rows by tiles of 16 columns, which a product takes as its
+    `row_norm` to read the RMS-normed stream without a norm kernel in between."""
+    _need_cuda(x, weight, bias, resid, norm_weight)
+    _rows2d("x", x)
+    _rows2d("resid", resid)
+    M, K = x.shape
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] != K or not weight.is_contiguous():
+        raise ValueError(f"linear_into_stream takes bfloat16 x [M, {K}] and a contiguous bfloat16 weight [N, {K}]")
+    if M > SKINNY_FAST_ROWS or K % 8 or x.stride(0) % 8:
+        raise ValueError("linear_into_stream: at most 32 rows, K and the row stride multiples of 8")
+    if resid.dtype != torch.float32 or tuple(resid.shape) != (M, N):
+        raise ValueError(f"the residual stream is float32 [{M}, {N}]")
+    if bias is not None and (bias.shape != (N,) or not bias.is_contiguous()):
+        raise ValueError(f"bias must be a contiguous [{N}] tensor")
+    if norm_weight is not None and (norm_weight.shape != (N,) or not norm_weight.is_contiguous()
+                                    or norm_weight.dtype not in (torch.float32, torch.bfloat16)):
+        raise ValueError(f"the norm weight is a contiguous float32 or bfloat16 [{N}] tensor")
+    scaled = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    partials = torch.empty(M, (N + 15) // 16, dtype=torch.float32, device=x.device)
+    check(load().fmsamd_gemm_skinny_residual_bf16(
+        x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
+        resid.data_ptr(), resid.stride(0), _ptr(norm_weight), _code(norm_weight.dtype) if norm_weight is not None else 0,
+        scaled.data_ptr(), scaled.stride(0), partials.data_ptr(), M, N, K, _row_scale(row_norm, M), _stream()))
+    return scaled, RowNorm(partials, eps)
+
+
 def gated_linear(
-    x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], activation: str, allow_library: bool = True
+    x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], activation: str, allow_library: bool = True,
+    row_norm: Optional[RowNorm] = None,
 ) -> torch.Tensor:
     """act(x Wg^T + bg) * (x Wu^T + bu) for weight = [Wg; Wu] stacked [2*hidden, K] -> [M, hidden]."""
     M = x.shape[0]
@@ -455,8 +523,11 @@ def gated_linear(
         out = torch.empty(M, hidden, dtype=torch.bfloat16, device=x.device)
         check(load().fmsamd_gemm_skinny_gated_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias),
                                                    _code(bias.dtype) if bias is not None else 0, out.data_ptr(), BF16,
-                                                   out.stride(0), M, hidden, K, ACTIVATIONS[activation], _stream()))
+                                                   out.stride(0), M, hidden, K, ACTIVATIONS[activation],
+                                                   _row_scale(row_norm, M), _stream()))
         return out
+    if row_norm is not None:
+        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 32 rows")
     gu = linear(x, weight, None, allow_library=allow_library)
     return gated_act(gu, bias, activation)
 

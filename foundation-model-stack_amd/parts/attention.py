@@ -17,7 +17,7 @@ import torch
 
 from ..cache import KVNeed
 from ..kernels import ops
-from .base import Mixer, Part, register_part
+from .base import BranchOutput, Mixer, Part, register_part, split_normed
 from .linear import Linear
 from .position import PositionEncoding
 
@@ -70,22 +70,33 @@ class MultiHeadAttention(Mixer):
             return 0  # the generic kernel takes tokens one by one
         return ops.prefill_qblock(self.nheads, self.kvheads, self.head_dim, n_tokens)
 
+    def _fused_decode(self, rows: int, dtype, batch) -> bool:
+        """True if projection, rotation and cache write of this step run as one kernel."""
+        rotates_by_table = self.position_encoder is None or self.position_encoder.rotary_tables() is not None
+        return (batch.is_decode and rows <= ops.QKV_ROPE_MAX_ROWS and dtype == torch.bfloat16
+                and self.qkv.w["weight"].dtype == torch.bfloat16 and self.head_dim % 16 == 0 and rotates_by_table)
+
+    def accepts_normed_rows(self, rows: int, dtype, batch) -> bool:
+        return self._fused_decode(rows, dtype, batch)
+
     def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
+        return self.forward_branch(x, batch, cache).value()
+
+    def forward_branch(self, x, batch, cache: LayerCache) -> BranchOutput:
+        x, row_norm = split_normed(x)
         H, K, D = self.nheads, self.kvheads, self.head_dim
         table = batch.block_tables[cache.group]
         tables = self.position_encoder.rotary_tables() if self.position_encoder is not None else None
         cos, sin, rot = tables if tables is not None else (None, None, 0)
         keys, values = (cache.keys, cache.values) if cache.owns else (None, None)
         weight = self.qkv.w["weight"]
-        fused = (
-            batch.is_decode and x.shape[0] <= ops.QKV_ROPE_MAX_ROWS and x.dtype == torch.bfloat16
-            and weight.dtype == torch.bfloat16 and D % 16 == 0 and (tables is not None or self.position_encoder is None)
-        )
-        if fused:
+        if self._fused_decode(x.shape[0], x.dtype, batch):
             # decode: projection, rotation and cache write in one kernel
             qkv = ops.qkv_rope_write(x, weight, self.qkv.w.get("bias"), batch.positions, batch.seq_of_token, table,
-                                     cos, sin, rot, keys, values, H, K, D)
+                                     cos, sin, rot, keys, values, H, K, D, row_norm=row_norm)
         else:
+            if row_norm is not None:
+                raise RuntimeError("a deferred norm reached a step that does not take one")
             qkv = self.qkv.forward(x)
             if tables is None and self.position_encoder is not None:
                 self.position_encoder.adjust_qk(qkv, batch, H, K, D)
@@ -97,7 +108,7 @@ class MultiHeadAttention(Mixer):
             decode=batch.is_decode, max_context=batch.max_context,
             qblock_start=qb_start, qblock_len=qb_len, qblock_tokens=size,
         )
-        return self.dense.forward(mixed)
+        return BranchOutput(mixed, self.dense)
 
 
 register_part("mixer", "attention", MultiHeadAttention)

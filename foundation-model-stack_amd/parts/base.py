@@ -63,6 +63,39 @@ class Part:
         """Called once after all parameters are bound: build tables, check what was bound."""
 
 
+class NormedRows:
+    """The input of a branch whose norm is left to the branch's first product: `rows` hold the stream times
+    the norm's weight in the activation type, `row_norm` what the product needs to divide by the rows' root
+    mean square (kernels.ops.RowNorm).  Only parts that say `accepts_normed_rows` ever see one."""
+
+    def __init__(self, rows: torch.Tensor, row_norm):
+        self.rows, self.row_norm = rows, row_norm
+
+    @property
+    def shape(self):
+        return self.rows.shape
+
+    @property
+    def dtype(self):
+        return self.rows.dtype
+
+
+class BranchOutput:
+    """A branch's output that is still one product away: linear(x).  Whoever holds the residual stream
+    decides whether that product also adds to the stream (ResidualStream.add_branch) or just runs."""
+
+    def __init__(self, x: torch.Tensor, linear: "Part"):
+        self.x, self.linear = x, linear
+
+    def value(self) -> torch.Tensor:
+        return self.linear.forward(self.x)
+
+
+def split_normed(x):
+    """(rows, row_norm) of a branch input, whether the norm was applied (row_norm None) or left to the product."""
+    return (x.rows, x.row_norm) if isinstance(x, NormedRows) else (x, None)
+
+
 class Mixer(Part):
     """A part that mixes information along the sequence.  It says what it needs of the cache:
     keys and values in pages (``kv_need``), fixed-size memory per sequence (``state_need``), or nothing."""
@@ -84,12 +117,27 @@ class Mixer(Part):
     def forward(self, x: torch.Tensor, batch, cache) -> torch.Tensor:
         raise NotImplementedError
 
+    # optional, for kernels that fuse across the boundary of the part --------
+    def accepts_normed_rows(self, rows: int, dtype, batch) -> bool:
+        """True if forward_branch takes a NormedRows for a step of this shape."""
+        return False
+
+    def forward_branch(self, x, batch, cache):
+        """Like forward, but may return a BranchOutput and may be given a NormedRows (if it says so)."""
+        return self.forward(x, batch, cache)
+
 
 class FeedForward(Part):
     """A part that maps every token on its own: [T, width] -> [T, width]."""
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
+
+    def accepts_normed_rows(self, rows: int, dtype) -> bool:
+        return False
+
+    def forward_branch(self, x):
+        return self.forward(x)
 
 
 # --------------------------------------------------------------------------

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from ..kernels import ops
-from .base import FeedForward, register_part
+from .base import BranchOutput, FeedForward, register_part, split_normed
 from .linear import Linear
 
 
@@ -24,8 +24,15 @@ class GatedLinearUnit(FeedForward):
         self.w2 = self.add_child("w2", Linear(self.hidden_dim, width, use_bias))
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        hidden = ops.gated_linear(x, self.wg1.w["weight"], self.wg1.w.get("bias"), self.activation)
-        return self.w2.forward(hidden)
+        return self.forward_branch(x).value()
+
+    def accepts_normed_rows(self, rows: int, dtype) -> bool:
+        return self.wg1.streams(rows, dtype)
+
+    def forward_branch(self, x) -> BranchOutput:
+        x, row_norm = split_normed(x)
+        hidden = ops.gated_linear(x, self.wg1.w["weight"], self.wg1.w.get("bias"), self.activation, row_norm=row_norm)
+        return BranchOutput(hidden, self.w2)
 
 
 register_part("feed_forward", "glu", GatedLinearUnit)

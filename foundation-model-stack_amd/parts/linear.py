@@ -19,5 +19,11 @@ class Linear(Part):
         if bias:
             self.declare("bias", (out_features,), init="zeros")
 
-    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-        return ops.linear(x, self.w["weight"], self.w.get("bias"), out_dtype=out_dtype)
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None, row_norm=None) -> torch.Tensor:
+        return ops.linear(x, self.w["weight"], self.w.get("bias"), out_dtype=out_dtype, row_norm=row_norm)
+
+    def streams(self, rows: int, dtype: torch.dtype) -> bool:
+        """True if a product of this shape runs in the weight-streaming kernel, which can take a deferred
+        row norm on its input and add its output into the residual stream."""
+        return dtype == torch.bfloat16 and self.w["weight"].dtype == torch.bfloat16 and rows <= ops.SKINNY_FAST_ROWS \
+            and self.in_features % 8 == 0

@@ -42,6 +42,11 @@ class ParameterizedNorm(Part):
         """resid += branch (float32, in place); returns norm(resid) in out_dtype (only `rows` if given)."""
         return ops.add_norm(resid, branch, self.w.get("weight"), self.w.get("bias"), self.eps, out_dtype, rows, self.use_mean)
 
+    def deferrable(self) -> bool:
+        """True if the norm is a row scale times a weight (no mean, no shift), so that a product can apply the
+        row scale to its result instead: (x / rms(x) * w) W^T = (x * w) W^T / rms(x)."""
+        return not self.use_mean and "bias" not in self.w
+
 
 register_part("norm", "rmsnorm", lambda width, eps=1e-6, **kw: ParameterizedNorm(width, eps, True, False, False, **kw))
 register_part("norm", "layernorm", lambda width, eps=1e-6, **kw: ParameterizedNorm(width, eps, True, True, True, **kw))

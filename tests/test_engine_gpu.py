@@ -336,6 +336,42 @@ def test_sampled_generation_is_batch_invariant(lib, folders):
     assert halves == together
 
 
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_decode_products_that_fuse_the_norms_change_only_rounding(lib, folders, name, monkeypatch):
+    """In bfloat16 decode steps the last product of a branch adds to the stream and prepares the next
+    norm's input.  The same steps with every norm as a kernel of its own give the same logits up to
+    rounding, and both follow the plain implementation."""
+    from fms_amd.engine import Engine
+    from fms_amd.kernels import ops
+    from fms_amd.parts import ResidualStream
+
+    calls = []
+    real = ops.linear_into_stream
+    monkeypatch.setattr(ops, "linear_into_stream", lambda *a, **k: (calls.append(1), real(*a, **k))[1])
+    cfg, weights = plain(folders, name)
+    model = get(lib, folders, name, "bfloat16")
+    lens = [40, 3, 17]
+    ids = [tokens_for(name, n + 6, 50 + n) for n in lens]
+    results = []
+    for fuse in (True, False):
+        monkeypatch.setattr(ResidualStream, "fuse_products", fuse)
+        engine = Engine(model, max_tokens=512, max_slots=3, use_graphs=False)
+        slots = [engine.new_sequence() for _ in lens]
+        engine.step(slots, [t[:n] for t, n in zip(ids, lens)], "last")
+        before = len(calls)
+        rows = [engine.step(slots, [[t[n + i]] for t, n in zip(ids, lens)], "last") for i in range(6)]
+        assert (len(calls) > before) == fuse
+        for s in slots:
+            engine.end_sequence(s)
+        results.append(torch.stack(rows).float().cpu())  # [6, 3, vocab]
+    fused, plain_norms = results
+    scale = float(plain_norms.abs().max())
+    assert float((fused - plain_norms).abs().max()) <= 0.02 * scale
+    for b, (t, n) in enumerate(zip(ids, lens)):
+        want = P.forward(weights, cfg, t)[n:]
+        check(fused[:, b], want, "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_graph_replay_equals_eager_steps(lib, folders, dtype, tmp_path):
     """Decode through captured graphs gives the tokens of eager steps: across page borders, when the

@@ -360,6 +360,80 @@ def test_gated_linear(ops, M, hidden, K):
             torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=4e-2, rtol=2e-2)))
 
 
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32])
+@pytest.mark.parametrize("N,K,eps", [(48, 24, 1e-5), (96, 176, 1e-6), (4096 + 40, 64, 1e-5), (100, 96, 1e-3)])
+def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
+    """The last product of a branch adds to the float32 stream and leaves the next norm's input; the
+    products that read it (plain, gated, qkv with rotation) finish the norm.  Against the plain formulas:
+    stream' = stream + x W^T + b;  y = rms_norm(stream') V^T."""
+    torch.manual_seed(12)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = (torch.randn(N, K) * 0.2).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16)
+    resid = torch.randn(M, N) * 3
+    resid[0] *= 40  # rows of very different size: a row scale applied to the wrong row shows
+    for norm_w in (torch.randn(N).abs().to(torch.bfloat16), torch.randn(N).abs(), None):
+        for bias in (None, b):
+            stream = dev(resid.clone())
+            scaled, row_norm = ops.linear_into_stream(dev(x), dev(w), None if bias is None else dev(bias), stream,
+                                                      None if norm_w is None else dev(norm_w), eps)
+            want_stream = resid.double() + x.double() @ w.double().t() + (0 if bias is None else bias.double())
+            torch.testing.assert_close(stream.cpu().double(), want_stream, atol=2e-3, rtol=1e-4)
+            got = stream.cpu()
+            assert row_norm.partials.shape == (M, (N + 15) // 16)
+            torch.testing.assert_close(row_norm.partials.cpu().sum(-1), got.pow(2).sum(-1), rtol=1e-5, atol=1e-5)
+            nw = torch.ones(N) if norm_w is None else norm_w.float()
+            torch.testing.assert_close(scaled.cpu().float(), (got * nw).to(torch.bfloat16).float(), atol=0, rtol=1e-2)
+            if N % 8:
+                continue
+            # consumers: what they make of (scaled, row_norm) against the product of the normed stream
+            normed = P.rms_norm(got, nw, eps)
+            N2 = 80
+            v = (torch.randn(N2, N) * 0.2).to(torch.bfloat16)
+            vb = torch.randn(N2).to(torch.bfloat16)
+            bound = dict(atol=0.02 * float((normed @ v.float().t()).abs().max()) + 1e-3, rtol=2e-2)
+            out = ops.linear(scaled, dev(v), dev(vb), row_norm=row_norm).cpu().float()
+            torch.testing.assert_close(out, normed @ v.float().t() + vb.float(), **bound)
+            out = ops.linear(scaled, dev(v), None, out_dtype=torch.float32, row_norm=row_norm).cpu()
+            torch.testing.assert_close(out, normed @ v.float().t(), **bound)
+            out = ops.gated_linear(scaled, dev(v), dev(vb), "swish", row_norm=row_norm).cpu().float()
+            gu = normed @ v.float().t() + vb.float()
+            want = P.silu(gu[:, :N2 // 2]) * gu[:, N2 // 2:]  # a product of two rounded values: its own scale
+            torch.testing.assert_close(out, want, atol=0.02 * float(want.abs().max()) + 1e-3, rtol=2e-2)
+            # the chain: a second product into the stream that reads the first one's rows
+            stream2 = dev(resid.clone())
+            w2 = (torch.randn(N, N) * 0.1).to(torch.bfloat16)
+            ops.linear_into_stream(scaled, dev(w2), None, stream2, None, eps, row_norm=row_norm)
+            torch.testing.assert_close(stream2.cpu(), resid + normed @ w2.float().t(), **bound)
+
+
+def test_qkv_rope_write_takes_a_deferred_row_norm(ops):
+    torch.manual_seed(13)
+    M, H, K, D, E, eps = 5, 4, 2, 32, 96, 1e-5
+    N = (H + 2 * K) * D
+    resid = torch.randn(M, E) * 2
+    resid[3] *= 30
+    nw = torch.randn(E).abs().to(torch.bfloat16)
+    x0 = torch.zeros(M, 8).to(torch.bfloat16)
+    stream = dev(resid.clone())
+    scaled, row_norm = ops.linear_into_stream(dev(x0), dev(torch.zeros(E, 8).to(torch.bfloat16)), None, stream, dev(nw), eps)
+    normed = ops.add_norm(dev(resid.clone()), None, dev(nw), None, eps, torch.bfloat16)
+    w = (torch.randn(N, E) * 0.2).to(torch.bfloat16)
+    positions = torch.randint(0, 200, (M,)).int()
+    seq = torch.arange(M).int()
+    table, n_pages = make_pages([256] * M, K, D, torch.bfloat16, seed=3)
+    cos, sin = ops.rope_table(dev(P.rope_frequencies(D, 10000.0)), 256)
+    res = []
+    for x, rn in ((normed, None), (scaled, row_norm)):
+        kc = torch.zeros(n_pages, K, PAGE, D, dtype=torch.bfloat16, device="cuda")
+        vc = torch.zeros(n_pages, K, D, PAGE, dtype=torch.bfloat16, device="cuda")
+        qkv = ops.qkv_rope_write(x, dev(w), None, dev(positions), dev(seq), dev(table), cos, sin, D, kc, vc, H, K, D, row_norm=rn)
+        res.append((qkv[:, : H * D].cpu().float(), kc.cpu().float(), vc.cpu().float()))
+    for a, b in zip(*res):
+        assert a.abs().max() > 0
+        torch.testing.assert_close(a, b, atol=0.02 * float(a.abs().max()), rtol=2e-2)
+
+
 # --------------------------------------------------------------------------
 def test_argmax(ops):
     torch.manual_seed(9)
