@@ -556,8 +556,22 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
   }
 }
 
+// The pages that split `split` of `n_splits` takes of a sequence whose visible keys are lo..pos: every
+// sequence's own pages are dealt out evenly, so that in a batch of unequal lengths every block has work in
+// proportion to its sequence.  Returns the number of splits that have pages at all (the first ones).
+__device__ __forceinline__ int split_pages(int lo, int pos, int n_splits, int split, int* page_lo, int* page_hi) {
+  const int first_page = lo / PAGE_TOKENS, last_page = pos / PAGE_TOKENS;
+  const int span = last_page - first_page + 1;
+  const int per = (span + n_splits - 1) / n_splits;
+  *page_lo = first_page + split * per;
+  *page_hi = *page_lo + per - 1 < last_page ? *page_lo + per - 1 : last_page;
+  return (span + per - 1) / per;
+}
+
 // Grid (split, kv head x head tile, token).  The waves of a block take the pages of its split in turn and
-// meet in LDS, so that a context of up to waves x pages_per_wave pages needs no second kernel.
+// meet in LDS; the splits of a token meet in the merge kernel.  (Merging in the block that finishes last,
+// behind a device-wide fence and a counter, was measured four times slower: the fence writes back and
+// invalidates the whole L2 of the block's XCD while the other blocks stream through it.)
 template <int MAXDT, int MAXW>
 __global__ void __launch_bounds__(MAXW* WAVE)
     attn_decode_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
@@ -565,7 +579,7 @@ __global__ void __launch_bounds__(MAXW* WAVE)
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                            int window, int pages_per_split, int tile_cols) {
+                            int window, int tile_cols) {
   extern __shared__ float lds[];  // [wave][tile_cols columns][head_dim + 2]
   const int split = blockIdx.x;
   const int group = nheads / kvheads;
@@ -589,20 +603,14 @@ __global__ void __launch_bounds__(MAXW* WAVE)
   }
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first_split = (lo / PAGE_TOKENS) / pages_per_split;
-  const int last_split = (pos / PAGE_TOKENS) / pages_per_split;
-  if (split < first_split || split > last_split) return;
+  int page_lo, page_hi;
+  if (split >= split_pages(lo, pos, n_splits, split, &page_lo, &page_hi)) return;
 
   const int* bt = block_table + (size_t)seq * table_stride;
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
 
   bf16x8 qreg[(MAXDT + 1) / 2];
   load_query<MAXDT>(qreg, r < cols ? q + (size_t)t * q_stride + (size_t)(head0 + r) * head_dim : nullptr, head_dim);
-
-  int page_lo = split * pages_per_split;
-  int page_hi = page_lo + pages_per_split - 1;
-  if (page_lo < lo / PAGE_TOKENS) page_lo = lo / PAGE_TOKENS;
-  if (page_hi > pos / PAGE_TOKENS) page_hi = pos / PAGE_TOKENS;
 
   WaveState<MAXDT, 1> st;
   wave_state_init(st);
@@ -667,20 +675,20 @@ __global__ void __launch_bounds__(MAXW* WAVE)
 __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          bf16* __restrict__ out, long out_stride, const int* __restrict__ positions,
                                          const int* __restrict__ seq_of_token, int nheads, int head_dim, int n_splits,
-                                         int window, int pages_per_split) {
+                                         int window) {
   const int h = blockIdx.x;
   const int t = blockIdx.y;
   if (seq_of_token[t] < 0) return;  // the decode kernel wrote zeros
   const int pos = positions[t];
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  const int first_split = (lo / PAGE_TOKENS) / pages_per_split;
-  const int last_split = (pos / PAGE_TOKENS) / pages_per_split;
+  int page_lo, page_hi;
+  const int active = split_pages(lo, pos, n_splits, 0, &page_lo, &page_hi);
   const size_t base = ((size_t)t * nheads + h) * n_splits;
   float m = -1e30f;
-  for (int s = first_split; s <= last_split; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
+  for (int s = 0; s < active; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
     float o = 0.f, l = 0.f;
-    for (int s = first_split; s <= last_split; ++s) {
+    for (int s = 0; s < active; ++s) {
       const float f = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m);  // maxima are base-2 logarithms
       o += f * part_o[(base + s) * head_dim + d];
       l += f * part_ml[(base + s) * 2 + 1];
@@ -825,7 +833,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   attn_decode_bf16_kernel<M, MAXW><<<grid, dim3(waves * WAVE), lds_bytes, stream>>>(                                 \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, pages_per_split, tile_cols)
+      window, tile_cols)
   if (head_dim <= 64)
     FMS_DC(4, 8);
   else if (head_dim <= 128)
@@ -837,8 +845,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   if (n_splits > 1) {
     dim3 mgrid(nheads, n_tokens);
     attn_decode_merge_kernel<<<mgrid, head_dim <= 64 ? 64 : 128, 0, stream>>>(
-        part_o, part_ml, (bf16*)out, out_stride, positions, seq_of_token, nheads, head_dim, n_splits, window,
-        pages_per_split);
+        part_o, part_ml, (bf16*)out, out_stride, positions, seq_of_token, nheads, head_dim, n_splits, window);
     FMS_LAUNCH_CHECK("attn_decode_merge");
   }
   return 0;

@@ -70,8 +70,10 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
                              int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
                              hipStream_t stream);
 
-// bfloat16 decode: one token per sequence.  A block of `waves` waves covers `pages_per_split` pages (its waves
-// take them in turn and merge in LDS); with more than one split a second kernel merges the partial results.
+// bfloat16 decode: one token per sequence.  The context bound max_context is cut into splits of
+// `pages_per_split` pages, and every sequence deals its own pages out evenly over that many blocks of `waves`
+// waves (which take them in turn and merge in LDS); with more than one split a second kernel merges the
+// partial results.
 long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits);
 int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_stride, void* workspace,
                             long workspace_bytes, const int* positions, const int* seq_of_token,

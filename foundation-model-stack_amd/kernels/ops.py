@@ -377,12 +377,15 @@ def decode_split(rows: int, n_pages: int):
     """(pages per split, waves per block) of the decode attention kernel.
 
     rows = tokens x kv heads.  A compute unit pulls only a small share of the memory bandwidth, so
-    the cache has to be spread over all of them: the context is cut into as many splits as give a
-    few hundred blocks; the waves of a block share its pages and merge in LDS, blocks of a row
-    merge in a second kernel.  With many rows one block takes the whole context."""
-    splits = max(1, min(-(-256 // max(rows, 1)), n_pages))
+    the cache has to be spread over all of them: the context bound is cut into as many splits as give
+    a few hundred blocks, and at least so many that a block has no more than 16 pages (every sequence
+    deals its own pages out evenly over the splits, so a long sequence among short ones does not end
+    up in one block).  The waves of a block share its pages and merge in LDS, the blocks of a row
+    merge in a second kernel."""
+    by_rows = min(-(-256 // max(rows, 1)), max(1, n_pages // 4))  # but no splits of under 4 pages
+    splits = max(1, min(max(by_rows, -(-n_pages // 16)), n_pages))
     pages = -(-n_pages // splits)
-    waves = max(1, min(8 if splits > 1 else 4, pages))
+    waves = max(1, min(8 if rows * splits <= 512 else 4, pages))
     return pages, waves
 
 
