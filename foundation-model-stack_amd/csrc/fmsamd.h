@@ -102,11 +102,13 @@ int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* 
 int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                   int out_dtype, long ldo, int M, int hidden, int K, int act,
                                   const fmsamd_row_scale* row_scale, hipStream_t stream);
-// resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, ceil(N/16)] = sums of
-// squares of resid by tiles of 16 columns.  At most 32 rows.
+// resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, partial_count] = sums
+// of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(N) says;
+// every entry is written).  At most 32 rows.
+int fmsamd_gemm_skinny_residual_partials(int N);
 int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                      float* resid, long ldr, const void* norm_w, int norm_w_dtype, void* scaled,
-                                     long ldo, float* partials, int M, int N, int K,
+                                     long ldo, float* partials, int partial_count, int M, int N, int K,
                                      const fmsamd_row_scale* row_scale, hipStream_t stream);
 
 // qkv = x W^T (+ bias) for at most 32 rows with the rotation and the cache write fused into the epilogue;

@@ -246,7 +246,7 @@ template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typena
 __global__ void __launch_bounds__(SK_WAVES* WAVE)
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
-                       RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
+                       int rows_per_block, RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
   constexpr bool GATED = EPI == EPI_GATED;
   __shared__ float red[SK_WAVES][NTB][MT][16][17];
   __shared__ int s_pos[MT * 16], s_seq[MT * 16], s_page[MT * 16];
@@ -254,7 +254,10 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
   const int wave = threadIdx.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  const int n0 = blockIdx.x * 16 * (GATED ? 1 : NTB);
+  // A block owns rows_per_block rows of W (a multiple of 8, at most 16 * NTB; its last tile may be partly
+  // empty): 24 rows make 256 equal blocks of 6144 rows where 16 would make 384.  Gated: 16 and 16.
+  const int n0 = blockIdx.x * (GATED ? 16 : rows_per_block);
+  const int n_end = GATED ? N : (n0 + rows_per_block < N ? n0 + rows_per_block : N);
 
   if (EPI == EPI_ROPE && threadIdx.x < MT * 16) {
     // index data of the rows, fetched while the weights stream
@@ -293,7 +296,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       const int n = n0 + ((idx >> 8) / MT) * 16 + (idx & 15);
       const int hh = n / rope.head_dim, d = n - hh * rope.head_dim;
       pre_resid[rd] = 1.f, pre_nw[rd] = 0.f;
-      if (idx < OUT_TILES * MT * 256 && m < M && n < N && hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr &&
+      if (idx < OUT_TILES * MT * 256 && m < M && n < n_end && hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr &&
           d < rope.rot_dim) {
         const int pos = rope.positions[m];
         const int tpos = pos < rope.max_pos ? pos : rope.max_pos - 1;  // the host has checked the range
@@ -308,7 +311,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       const int idx = threadIdx.x + rd * SK_WAVES * WAVE;
       const int m = ((idx >> 8) % MT) * 16 + ((idx >> 4) & 15);
       const int n = n0 + ((idx >> 8) / MT) * 16 + (idx & 15);
-      const bool live = idx < OUT_TILES * MT * 256 && m < M && n < N;
+      const bool live = idx < OUT_TILES * MT * 256 && m < M && n < n_end;
       pre_resid[rd] = live ? res.resid[(size_t)m * res.ldr + n] : 0.f;
       pre_nw[rd] = 1.f;
       if (live && res.norm_w != nullptr)
@@ -321,7 +324,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 #pragma unroll
   for (int t = 0; t < NTB; ++t) {
     const int n = n0 + (t == 0 ? 0 : (GATED ? tile2_offset : 16 * t)) + r;
-    const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : N;
+    const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : n_end;
     wok[t] = n < limit;
     wrow[t] = w + (size_t)(wok[t] ? n : 0) * K;
   }
@@ -412,7 +415,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
     const int ti = (idx >> 8) / MT;    // n tile
     const int m = tj * 16 + mm;
     const int n = n0 + ti * 16 + nn;
-    const bool live = m < M && n < N;
+    const bool live = m < M && n < n_end;
     float v = 0.f;
 #pragma unroll
     for (int wv = 0; wv < SK_WAVES; ++wv) v += red[wv][ti][tj][nn][mm];
@@ -465,7 +468,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       float sq = stream * stream;
 #pragma unroll
       for (int off = 8; off > 0; off >>= 1) sq += __shfl_xor(sq, off, WAVE);
-      if (nn == 0 && m < M && n0 + ti * 16 < N) res.partials[(size_t)m * res.tiles + blockIdx.x * NTB + ti] = sq;
+      if (nn == 0 && m < M) res.partials[(size_t)m * res.tiles + blockIdx.x * NTB + ti] = sq;  // 0 for an empty tile
     } else {
       if (!live) continue;
       if (bias) v += to_f32(bias[n]);
@@ -476,15 +479,17 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 
 template <int NTB, int MT, int EPI>
 static void launch_skinny(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
-                          int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int blocks,
+                          int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int rows_per_block,
                           hipStream_t stream, RowScale scale, RopeEpilogue rope = RopeEpilogue{},
                           ResidEpilogue res = ResidEpilogue{}) {
+  const int blocks = ceil_div(N, EPI == EPI_GATED ? 16 : rows_per_block);
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
   constexpr int SK_WAVES = NTB * MT > 4 ? 4 : 8;
   constexpr int UNR = (NTB + MT) <= 2 ? 4 : ((NTB + MT) <= 4 ? 2 : 1);
 #define FMS_SK(O, B)                                                                                 \
   skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, EPI, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(     \
-      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, scale, rope, res)
+      (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, rows_per_block,  \
+      scale, rope, res)
   if (out_dtype == FMS_BF16) {
     if (fb)
       FMS_SK(bf16, float);
@@ -497,6 +502,21 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
       FMS_SK(float, bf16);
   }
 #undef FMS_SK
+}
+
+// Rows of W per block (16, 24 or 32) for a product of N rows: the choice that costs the fewest rounds of
+// blocks over the compute units, a round costing as much as its blocks have rows.  Large products take 32
+// (the activations are then read once per two tiles).
+#define SK_COMPUTE_UNITS 256
+static int skinny_rows_per_block(int N) {
+  if (N >= 16384) return 32;
+  int best = 16;
+  long best_cost = 0;
+  for (int rows = 16; rows <= 32; rows += 8) {
+    const long cost = (long)ceil_div(ceil_div(N, rows), SK_COMPUTE_UNITS) * rows;
+    if (rows == 16 || cost < best_cost) best = rows, best_cost = cost;
+  }
+  return best;
 }
 
 // Checks a deferred row norm and turns it into the kernel's argument.
@@ -520,12 +540,10 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   FMS_REQUIRE(ldx >= K && ldo >= N, "gemm_skinny_bf16: leading dimensions too small");
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_bf16: unknown output dtype %d", out_dtype);
   const int mt = ceil_div(M, 16);
-  // two tiles per block when that still leaves every CU several blocks
-  const bool two = N >= 16384;
-  const int blocks = ceil_div(N, two ? 32 : 16);
+  const int rows = skinny_rows_per_block(N);
 #define FMS_LS(NTB, MT) \
-  launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, blocks, stream, scale)
-  if (two) {
+  launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, rows, stream, scale)
+  if (rows > 16) {
     if (mt == 1) FMS_LS(2, 1); else if (mt == 2) FMS_LS(2, 2); else if (mt == 3) FMS_LS(2, 3); else FMS_LS(2, 4);
   } else {
     if (mt == 1) FMS_LS(1, 1); else if (mt == 2) FMS_LS(1, 2); else if (mt == 3) FMS_LS(1, 3); else FMS_LS(1, 4);
@@ -550,9 +568,8 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_gated_bf16: unknown output dtype %d", out_dtype);
   FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gemm_skinny_gated_bf16: unknown activation %d", act);
   const int mt = ceil_div(M, 16);
-  const int blocks = ceil_div(hidden, 16);
 #define FMS_LG(MT) \
-  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, blocks, \
+  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, 16, \
                                   stream, scale)
   if (mt == 1) FMS_LG(1); else if (mt == 2) FMS_LG(2); else if (mt == 3) FMS_LG(3); else FMS_LG(4);
 #undef FMS_LG
@@ -585,13 +602,15 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   FMS_REQUIRE(cos_t == nullptr || (max_pos > 0 && sin_t != nullptr), "qkv_rope_skinny_bf16: empty rotary table");
   RopeEpilogue rope{positions, seq_of_token, block_table, table_stride, rot_dim > 0 ? cos_t : nullptr, sin_t, rot_dim,
                     max_pos, (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim};
-  const int blocks = N / 16;
-  if (M <= 16)
-    launch_skinny<1, 1, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
-                                  rope);
-  else
-    launch_skinny<1, 2, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
-                                  rope);
+  const int rows = skinny_rows_per_block(N);
+#define FMS_LR(NTB, MT) \
+  launch_skinny<NTB, MT, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
+  if (rows > 16) {
+    if (M <= 16) FMS_LR(2, 1); else FMS_LR(2, 2);
+  } else {
+    if (M <= 16) FMS_LR(1, 1); else FMS_LR(1, 2);
+  }
+#undef FMS_LR
   FMS_LAUNCH_CHECK("qkv_rope_skinny_bf16");
   return 0;
 }
@@ -600,13 +619,20 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
 //   resid[M, N] += x w^T (+ bias)                      float32, in place
 //   scaled[M, N] = resid * norm_w                      bfloat16: the next norm's input, not yet divided by its
 //                                                      root mean square
-//   partials[m, i] = sum over columns 16 i .. 16 i + 15 of resid[m]^2      [M, ceil(N / 16)]
+//   partials[m, i] = sums of resid[m]^2 over groups of up to 16 columns, the unused ones zero
+//                    [M, partial_count], partial_count >= fmsamd_gemm_skinny_residual_partials(N)
 // A product that takes `scaled` with these partials as its deferred row norm then equals the product of the
 // normed stream.  M <= 32.
+extern "C" int fmsamd_gemm_skinny_residual_partials(int N) {
+  const int rows = skinny_rows_per_block(N);
+  return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
+}
+
 extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias,
                                                 int bias_dtype, float* resid, long ldr, const void* norm_w,
-                                                int norm_w_dtype, void* scaled, long ldo, float* partials, int M, int N,
-                                                int K, const fmsamd_row_scale* row_scale, hipStream_t stream) {
+                                                int norm_w_dtype, void* scaled, long ldo, float* partials,
+                                                int partial_count, int M, int N, int K,
+                                                const fmsamd_row_scale* row_scale, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   FMS_REQUIRE(M > 0 && M <= 32 && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 32)", M, N, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_residual_bf16: K=%d and the row stride %ld must be multiples of 8",
@@ -617,14 +643,20 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
   FMS_REQUIRE(resid != nullptr && scaled != nullptr && partials != nullptr, "gemm_skinny_residual_bf16: null buffer");
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
-  const int blocks = ceil_div(N, 16);
-  ResidEpilogue res{resid, ldr, norm_w, norm_w_dtype == FMS_F32, partials, blocks};
-  if (M <= 16)
-    launch_skinny<1, 1, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
-                                   RopeEpilogue{}, res);
-  else
-    launch_skinny<1, 2, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, blocks, stream, scale,
-                                   RopeEpilogue{}, res);
+  const int rows = skinny_rows_per_block(N);
+  const int tiles = ceil_div(N, rows) * (rows > 16 ? 2 : 1);
+  FMS_REQUIRE(partial_count >= tiles, "gemm_skinny_residual_bf16: room for %d partial sums per row, %d needed",
+              partial_count, tiles);
+  ResidEpilogue res{resid, ldr, norm_w, norm_w_dtype == FMS_F32, partials, partial_count};
+#define FMS_LX(NTB, MT)                                                                                              \
+  launch_skinny<NTB, MT, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, \
+                                    scale, RopeEpilogue{}, res)
+  if (rows > 16) {
+    if (M <= 16) FMS_LX(2, 1); else FMS_LX(2, 2);
+  } else {
+    if (M <= 16) FMS_LX(1, 1); else FMS_LX(1, 2);
+  }
+#undef FMS_LX
   FMS_LAUNCH_CHECK("gemm_skinny_residual_bf16");
   return 0;
 }

@@ -41,7 +41,8 @@ _SIGNATURES = {
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
     "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P, P],
     "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P, P],
-    "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, P, P],
+    "fmsamd_gemm_skinny_residual_partials": [I],
+    "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
 }

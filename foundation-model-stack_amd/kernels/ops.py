@@ -496,11 +496,13 @@ def linear_into_stream(
                                     or norm_weight.dtype not in (torch.float32, torch.bfloat16)):
         raise ValueError(f"the norm weight is a contiguous float32 or bfloat16 [{N}] tensor")
     scaled = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
-    partials = torch.empty(M, (N + 15) // 16, dtype=torch.float32, device=x.device)
-    check(load().fmsamd_gemm_skinny_residual_bf16(
+    lib = load()
+    partials = torch.empty(M, lib.fmsamd_gemm_skinny_residual_partials(N), dtype=torch.float32, device=x.device)
+    check(lib.fmsamd_gemm_skinny_residual_bf16(
         x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
         resid.data_ptr(), resid.stride(0), _ptr(norm_weight), _code(norm_weight.dtype) if norm_weight is not None else 0,
-        scaled.data_ptr(), scaled.stride(0), partials.data_ptr(), M, N, K, _row_scale(row_norm, M), _stream()))
+        scaled.data_ptr(), scaled.stride(0), partials.data_ptr(), partials.shape[1], M, N, K, _row_scale(row_norm, M),
+        _stream()))
     return scaled, RowNorm(partials, eps)
 
 

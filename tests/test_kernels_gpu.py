@@ -186,7 +186,7 @@ def test_rope_kv_write(ops, dtype, H, K, D, rot):
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 32])
-@pytest.mark.parametrize("H,K,D,rot,E", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 40), (8, 8, 32, 16, 256)])
+@pytest.mark.parametrize("H,K,D,rot,E", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 40), (8, 8, 32, 16, 256), (40, 4, 128, 128, 32), (30, 2, 136, 136, 32)])
 def test_qkv_rope_write_equals_the_separate_kernels(ops, M, H, K, D, rot, E):
     """The decode-time fusion (projection + rotation + cache write) against linear followed by rope_kv_write."""
     torch.manual_seed(11)
@@ -361,7 +361,7 @@ def test_gated_linear(ops, M, hidden, K):
 
 
 @pytest.mark.parametrize("M", [1, 7, 16, 17, 32])
-@pytest.mark.parametrize("N,K,eps", [(48, 24, 1e-5), (96, 176, 1e-6), (4096 + 40, 64, 1e-5), (100, 96, 1e-3)])
+@pytest.mark.parametrize("N,K,eps", [(48, 24, 1e-5), (96, 176, 1e-6), (4096 + 40, 64, 1e-5), (100, 96, 1e-3), (6144, 32, 1e-5)])
 def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
     """The last product of a branch adds to the float32 stream and leaves the next norm's input; the
     products that read it (plain, gated, qkv with rotation) finish the norm.  Against the plain formulas:
@@ -380,7 +380,6 @@ def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
             want_stream = resid.double() + x.double() @ w.double().t() + (0 if bias is None else bias.double())
             torch.testing.assert_close(stream.cpu().double(), want_stream, atol=2e-3, rtol=1e-4)
             got = stream.cpu()
-            assert row_norm.partials.shape == (M, (N + 15) // 16)
             torch.testing.assert_close(row_norm.partials.cpu().sum(-1), got.pow(2).sum(-1), rtol=1e-5, atol=1e-5)
             nw = torch.ones(N) if norm_w is None else norm_w.float()
             torch.testing.assert_close(scaled.cpu().float(), (got * nw).to(torch.bfloat16).float(), atol=0, rtol=1e-2)
