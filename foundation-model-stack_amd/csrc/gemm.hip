@@ -6,9 +6,9 @@
 //   * gemm_bf16_kernel: bfloat16 in, MFMA 16x16x32 with float32 accumulation,
 //     bfloat16 or float32 out; LDS-tiled 128x128x32.  Any M and N; K % 8 == 0.
 //   * skinny_bf16_kernel: M <= 64 rows of x (decode).  Weight-streaming: a
-//     block owns one or two 16-row tiles of W, its waves split K, operands go
-//     from global memory straight into MFMA registers, partial sums meet in
-//     LDS.  Optional fused gate: out = act(x Wg^T) * (x Wu^T).
+//     block owns one or two 16-row tiles of W, its waves split K, loads take
+//     long contiguous runs and change to the MFMA layout in LDS, partial
+//     sums meet in LDS.  Optional fused gate: out = act(x Wg^T) * (x Wu^T).
 #include "common.h"
 #include "fmsamd.h"
 
@@ -239,16 +239,19 @@ struct RopeEpilogue {
 
 // NTB: 16-row tiles of W per block (the second tile starts `tile2_offset` rows after the first).
 // MT : 16-row tiles of x.
-// SK_WAVES: waves of a block (8, or 4 when NTB*MT > 4 so that the LDS buffer stays under 64 KB).
-// UNR: chunks of 64 k-values whose loads a wave issues before it multiplies: what keeps enough
-// bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 2 loads of 16 bytes outstanding).
+// SK_WAVES: waves of a block.
+// UNR: groups of 128 k-values whose loads a wave issues before it multiplies: what keeps enough
+// bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 4 loads of 16 bytes outstanding).
 template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typename BiasT>
 __global__ void __launch_bounds__(SK_WAVES* WAVE)
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
                        int rows_per_block, RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
   constexpr bool GATED = EPI == EPI_GATED;
-  __shared__ float red[SK_WAVES][NTB][MT][16][17];
+  // per wave: one tile of 16 rows x 128 k (4 KB) of W and one of x between load and MFMA layout; after
+  // the stream the region holds the wave's partial output tiles
+  constexpr int STAGE_BYTES = NTB * MT * 16 * 17 * 4 > 8192 ? NTB * MT * 16 * 17 * 4 : 8192;
+  __shared__ __attribute__((aligned(16))) unsigned char stage[SK_WAVES * STAGE_BYTES];
   __shared__ int s_pos[MT * 16], s_seq[MT * 16], s_page[MT * 16];
   __shared__ float s_scale[MT * 16];
   const int wave = threadIdx.x / WAVE;
@@ -319,22 +322,18 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
     }
   }
 
-  const bf16* wrow[NTB];
-  bool wok[NTB];
-#pragma unroll
-  for (int t = 0; t < NTB; ++t) {
-    const int n = n0 + (t == 0 ? 0 : (GATED ? tile2_offset : 16 * t)) + r;
-    const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : n_end;
-    wok[t] = n < limit;
-    wrow[t] = w + (size_t)(wok[t] ? n : 0) * K;
-  }
-  const bf16* xrow[MT];
-  bool xok[MT];
-#pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    xok[t] = t * 16 + r < M;
-    xrow[t] = x + (size_t)(xok[t] ? t * 16 + r : 0) * ldx;
-  }
+  // ---- the weight stream --------------------------------------------------
+  // K in groups of 128.  A load instruction takes 4 rows x 256 contiguous bytes (16 lanes of 16 bytes a
+  // row): runs that long are what the memory system streams at full rate, where the MFMA operand layout
+  // (16 rows x 64 bytes) reaches two thirds of it.  The group goes through the wave's own LDS region to
+  // change layout: written as loaded, read back as MFMA operands (lane (r, g) takes row r, k-step s at
+  // 16-byte piece 4 s + g).  Pieces are XOR-swizzled with the row so that both directions spread over
+  // the banks.  Weights are loaded non-temporally: they are read once.
+  const int lrow = lane >> 4, seg = lane & 15;
+  bf16* const stage_w = reinterpret_cast<bf16*>(stage + (size_t)wave * STAGE_BYTES);
+  bf16* const stage_x = stage_w + 2048;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  for (int i = lane; i < 256; i += WAVE) *reinterpret_cast<bf16x8*>(stage_x + i * 8) = zero;
 
   f32x4 acc[NTB][MT];
 #pragma unroll
@@ -342,44 +341,85 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 #pragma unroll
     for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // K in chunks of 64: lane group g covers k = chunk*64 + g*16 .. +16 (two MFMA steps).
-  // A wave takes UNR neighbouring chunks at a time.
-  const int nchunks = (K + 63) / 64;
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-  for (int ch0 = wave * UNR; ch0 < nchunks; ch0 += SK_WAVES * UNR) {
-    bf16x8 wa[UNR][NTB], wb[UNR][NTB], xa[UNR][MT], xb[UNR][MT];
+  const int ngroups = (K + 127) / 128;
+  for (int c0 = wave * UNR; c0 < ngroups; c0 += SK_WAVES * UNR) {
+    bf16x8 wreg[UNR][NTB][4], xreg[UNR][MT][4];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
-      const int k = (ch0 + u) * 64 + g * 16;
+      const int k = (c0 + u) * 128 + seg * 8;
+      const bool kok = k < K;
 #pragma unroll
       for (int t = 0; t < NTB; ++t) {
-        wa[u][t] = (wok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k) : zero;
-        wb[u][t] = (wok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(wrow[t] + k + 8) : zero;
+        const int nbase = n0 + (t == 0 ? 0 : (GATED ? tile2_offset : 16 * t));
+        const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : n_end;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int n = nbase + 4 * q + lrow;
+          wreg[u][t][q] = (kok && n < limit)
+                              ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w + (size_t)n * K + k))
+                              : zero;
+        }
       }
 #pragma unroll
-      for (int t = 0; t < MT; ++t) {
-        xa[u][t] = (xok[t] && k < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k) : zero;
-        xb[u][t] = (xok[t] && k + 8 < K) ? *reinterpret_cast<const bf16x8*>(xrow[t] + k + 8) : zero;
-      }
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int m = t * 16 + 4 * q + lrow;
+          if (t * 16 + 4 * q < M)  // uniform: whole instructions fall away for few rows
+            xreg[u][t][q] = (kok && m < M) ? *reinterpret_cast<const bf16x8*>(x + (size_t)m * ldx + k) : zero;
+        }
     }
 #pragma unroll
-    for (int u = 0; u < UNR; ++u)
+    for (int u = 0; u < UNR; ++u) {
+      if (c0 + u >= ngroups) break;  // uniform
+      // the wave's two 4 KB regions are its own: LDS operations of one wave keep their order, so a tile
+      // may overwrite the one before it as soon as that one's reads are issued
+      bf16x8 a[NTB][4];
 #pragma unroll
-      for (int i = 0; i < NTB; ++i)
+      for (int t = 0; t < NTB; ++t) {
 #pragma unroll
-        for (int j = 0; j < MT; ++j) {
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u][i], xa[u][j], acc[i][j], 0, 0, 0);
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wb[u][i], xb[u][j], acc[i][j], 0, 0, 0);
+        for (int q = 0; q < 4; ++q) {
+          const int row = 4 * q + lrow;
+          *reinterpret_cast<bf16x8*>(stage_w + row * 128 + ((seg ^ row) & 15) * 8) = wreg[u][t][q];
         }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int st = 0; st < 4; ++st)
+          a[t][st] = *reinterpret_cast<const bf16x8*>(stage_w + r * 128 + (((st * 4 + g) ^ r) & 15) * 8);
+        __builtin_amdgcn_wave_barrier();
+      }
+#pragma unroll
+      for (int j = 0; j < MT; ++j) {
+        if (j * 16 >= M) break;  // uniform: the tile has no rows, its sums stay zero
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int row = 4 * q + lrow;
+          const bool loaded = j * 16 + 4 * q < M;  // uniform
+          if (MT == 1 && !loaded) continue;        // one tile only: its empty rows were zeroed at the start
+          *reinterpret_cast<bf16x8*>(stage_x + row * 128 + ((seg ^ row) & 15) * 8) = loaded ? xreg[u][j][q] : zero;
+        }
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int st = 0; st < 4; ++st) {
+          const bf16x8 bx = *reinterpret_cast<const bf16x8*>(stage_x + r * 128 + (((st * 4 + g) ^ r) & 15) * 8);
+#pragma unroll
+          for (int i = 0; i < NTB; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i][st], bx, acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+    }
   }
 
-  // partial tiles meet in LDS: red[wave][tile n][tile m][n row][m column]
+  // partial tiles meet in LDS, each wave's in its own region: [tile n][tile m][n row][m column (17)]
+  {
+    float* red_w = reinterpret_cast<float*>(stage + (size_t)wave * STAGE_BYTES);
 #pragma unroll
-  for (int i = 0; i < NTB; ++i)
+    for (int i = 0; i < NTB; ++i)
 #pragma unroll
-    for (int j = 0; j < MT; ++j)
+      for (int j = 0; j < MT; ++j)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) red[wave][i][j][g * 4 + e][r] = acc[i][j][e];
+        for (int e = 0; e < 4; ++e) red_w[((i * MT + j) * 16 + g * 4 + e) * 17 + r] = acc[i][j][e];
+  }
 
   if (scale.partials != nullptr) {
     // the rows' scales: partial sums in a fixed order, the same bits whatever the launch looks like
@@ -418,14 +458,16 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
     const bool live = m < M && n < n_end;
     float v = 0.f;
 #pragma unroll
-    for (int wv = 0; wv < SK_WAVES; ++wv) v += red[wv][ti][tj][nn][mm];
+    for (int wv = 0; wv < SK_WAVES; ++wv)
+      v += reinterpret_cast<const float*>(stage + (size_t)wv * STAGE_BYTES)[((ti * MT + tj) * 16 + nn) * 17 + mm];
     const float row_scale = (scale.partials != nullptr && m < M) ? s_scale[m] : 1.f;
     v *= row_scale;
     if (EPI == EPI_GATED) {
       if (!live) continue;
       float u = 0.f;
 #pragma unroll
-      for (int wv = 0; wv < SK_WAVES; ++wv) u += red[wv][1][tj][nn][mm];
+      for (int wv = 0; wv < SK_WAVES; ++wv)
+        u += reinterpret_cast<const float*>(stage + (size_t)wv * STAGE_BYTES)[((1 * MT + tj) * 16 + nn) * 17 + mm];
       u *= row_scale;
       if (bias) {
         v += to_f32(bias[n]);
@@ -484,8 +526,8 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
                           ResidEpilogue res = ResidEpilogue{}) {
   const int blocks = ceil_div(N, EPI == EPI_GATED ? 16 : rows_per_block);
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
-  constexpr int SK_WAVES = NTB * MT > 4 ? 4 : 8;
-  constexpr int UNR = (NTB + MT) <= 2 ? 4 : ((NTB + MT) <= 4 ? 2 : 1);
+  constexpr int SK_WAVES = 8;
+  constexpr int UNR = (NTB + MT) <= 2 ? 2 : 1;
 #define FMS_SK(O, B)                                                                                 \
   skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, EPI, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(     \
       (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, rows_per_block,  \
