@@ -104,14 +104,14 @@ int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const 
                                   const fmsamd_row_scale* row_scale, hipStream_t stream);
 // resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, partial_count] = sums
 // of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(N) says;
-// every entry is written).  At most 32 rows.
+// every entry is written).  At most 64 rows.
 int fmsamd_gemm_skinny_residual_partials(int N);
 int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                      float* resid, long ldr, const void* norm_w, int norm_w_dtype, void* scaled,
                                      long ldo, float* partials, int partial_count, int M, int N, int K,
                                      const fmsamd_row_scale* row_scale, hipStream_t stream);
 
-// qkv = x W^T (+ bias) for at most 32 rows with the rotation and the cache write fused into the epilogue;
+// qkv = x W^T (+ bias) for at most 64 rows with the rotation and the cache write fused into the epilogue;
 // only the query columns of `out` are written
 int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                 long ldo, int M, int K, const int* positions, const int* seq_of_token,

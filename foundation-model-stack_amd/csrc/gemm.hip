@@ -621,7 +621,7 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
 
 // qkv[M, (H+2K)*D] = x W^T (+ bias) with the rotation of q and k and the cache write of k and v fused into
 // the epilogue: the decode-time twin of fmsamd_gemm_skinny_bf16 followed by fmsamd_rope_kv_write.  Only the
-// query columns of `out` are written.  M <= 32.
+// query columns of `out` are written.  M <= 64.
 extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                            void* out, long ldo, int M, int K, const int* positions,
                                            const int* seq_of_token, const int* block_table, int table_stride,
@@ -632,8 +632,8 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   const int N = (nheads + 2 * kvheads) * head_dim;
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
-  FMS_REQUIRE(M > 0 && M <= 32 && K > 0 && nheads > 0 && kvheads > 0 && head_dim > 0,
-              "qkv_rope_skinny_bf16: bad sizes M=%d K=%d (M <= 32)", M, K);
+  FMS_REQUIRE(M > 0 && M <= 64 && K > 0 && nheads > 0 && kvheads > 0 && head_dim > 0,
+              "qkv_rope_skinny_bf16: bad sizes M=%d K=%d (M <= 64)", M, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "qkv_rope_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N, "qkv_rope_skinny_bf16: leading dimensions too small");
   FMS_REQUIRE(head_dim % 2 == 0 && N % 16 == 0, "qkv_rope_skinny_bf16: head size %d must be even and the row a multiple of 16",
@@ -645,12 +645,13 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   RopeEpilogue rope{positions, seq_of_token, block_table, table_stride, rot_dim > 0 ? cos_t : nullptr, sin_t, rot_dim,
                     max_pos, (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim};
   const int rows = skinny_rows_per_block(N);
+  const int mt = ceil_div(M, 16);
 #define FMS_LR(NTB, MT) \
   launch_skinny<NTB, MT, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
   if (rows > 16) {
-    if (M <= 16) FMS_LR(2, 1); else FMS_LR(2, 2);
+    if (mt == 1) FMS_LR(2, 1); else if (mt == 2) FMS_LR(2, 2); else if (mt == 3) FMS_LR(2, 3); else FMS_LR(2, 4);
   } else {
-    if (M <= 16) FMS_LR(1, 1); else FMS_LR(1, 2);
+    if (mt == 1) FMS_LR(1, 1); else if (mt == 2) FMS_LR(1, 2); else if (mt == 3) FMS_LR(1, 3); else FMS_LR(1, 4);
   }
 #undef FMS_LR
   FMS_LAUNCH_CHECK("qkv_rope_skinny_bf16");
@@ -664,7 +665,7 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
 //   partials[m, i] = sums of resid[m]^2 over groups of up to 16 columns, the unused ones zero
 //                    [M, partial_count], partial_count >= fmsamd_gemm_skinny_residual_partials(N)
 // A product that takes `scaled` with these partials as its deferred row norm then equals the product of the
-// normed stream.  M <= 32.
+// normed stream.  M <= 64.
 extern "C" int fmsamd_gemm_skinny_residual_partials(int N) {
   const int rows = skinny_rows_per_block(N);
   return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
@@ -676,7 +677,7 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
                                                 int partial_count, int M, int N, int K,
                                                 const fmsamd_row_scale* row_scale, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  FMS_REQUIRE(M > 0 && M <= 32 && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 32)", M, N, K);
+  FMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_residual_bf16: K=%d and the row stride %ld must be multiples of 8",
               K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N && ldr >= N, "gemm_skinny_residual_bf16: leading dimensions too small");
@@ -690,13 +691,14 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
   FMS_REQUIRE(partial_count >= tiles, "gemm_skinny_residual_bf16: room for %d partial sums per row, %d needed",
               partial_count, tiles);
   ResidEpilogue res{resid, ldr, norm_w, norm_w_dtype == FMS_F32, partials, partial_count};
+  const int mt = ceil_div(M, 16);
 #define FMS_LX(NTB, MT)                                                                                              \
   launch_skinny<NTB, MT, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, \
                                     scale, RopeEpilogue{}, res)
   if (rows > 16) {
-    if (M <= 16) FMS_LX(2, 1); else FMS_LX(2, 2);
+    if (mt == 1) FMS_LX(2, 1); else if (mt == 2) FMS_LX(2, 2); else if (mt == 3) FMS_LX(2, 3); else FMS_LX(2, 4);
   } else {
-    if (M <= 16) FMS_LX(1, 1); else FMS_LX(1, 2);
+    if (mt == 1) FMS_LX(1, 1); else if (mt == 2) FMS_LX(1, 2); else if (mt == 3) FMS_LX(1, 3); else FMS_LX(1, 4);
   }
 #undef FMS_LX
   FMS_LAUNCH_CHECK("gemm_skinny_residual_bf16");

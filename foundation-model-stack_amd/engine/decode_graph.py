@@ -15,6 +15,8 @@ used when every part of the model says it can be captured.
 
 from __future__ import annotations
 
+import gc
+
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -24,7 +26,8 @@ from ..kernels import ops
 from .batch import StepBatch
 
 ROW_BUCKETS = (1, 2, 4, 8, 16, 24, 32, 48, 64, 96, 128, 192, 256)
-CONTEXT_BUCKET = 1024
+CONTEXT_BUCKET = 2048  # the smallest context bound of a graph; larger ones double
+CONTEXT_HEADROOM = 256  # a new graph is captured for a bound this far beyond the longest context
 
 
 def row_bucket(n: int) -> int:
@@ -35,7 +38,13 @@ def row_bucket(n: int) -> int:
 
 
 def context_bucket(n: int, limit: int) -> int:
-    return min(-(-n // CONTEXT_BUCKET) * CONTEXT_BUCKET, max(limit, 1))
+    """The context bound of the graph captured for contexts of up to n tokens: a power of two times 2048,
+    at most `limit`.  The decode attention deals every sequence's own pages out over its splits, so a bound
+    well above the contexts costs little, and doubling keeps the number of captures small."""
+    bound = CONTEXT_BUCKET
+    while bound < n:
+        bound *= 2
+    return min(bound, max(limit, 1))
 
 
 class DecodeGraph:
@@ -80,9 +89,19 @@ class DecodeGraph:
             self._run()  # warm-up: lazy initialisation and allocator growth happen outside the capture
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph):
-            self._run()
+        # No garbage collection while the stream is capturing: a collector pass that finds an old engine's
+        # graphs (they sit in reference cycles) would destroy them in the middle of the capture, which the
+        # runtime refuses, and the refusal inside a destructor ends the process.  Collect before, not during.
+        gc.collect()
+        was_enabled = gc.isenabled()
+        gc.disable()
+        try:
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self._run()
+        finally:
+            if was_enabled:
+                gc.enable()
         torch.cuda.synchronize()
 
     def load(self, slots: Sequence[int], tokens: Sequence[int], positions: Sequence[int], seeds, counters) -> None:

@@ -19,7 +19,7 @@ from ..cache import CacheFull, pages_for
 from ..kernels import ops
 from ..sampling import SamplingParams, choose
 from .batch import StepBatch, build_batch
-from .decode_graph import DecodeGraph, context_bucket, row_bucket
+from .decode_graph import CONTEXT_HEADROOM, DecodeGraph, context_bucket, row_bucket
 from .model import DecoderModel
 
 
@@ -44,6 +44,7 @@ class Engine:
             use_graphs = not os.environ.get("FMS_AMD_NO_GRAPHS")
         self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", True) for p in model.walk())
         self._graphs = {}
+        self.graph_captures = []  # (rows, context bound) of every capture, in order
 
     # ---- sequences ---------------------------------------------------------
     def new_sequence(self) -> int:
@@ -102,14 +103,18 @@ class Engine:
                 raise IndexError(f"sequence in slot {s} has reached the model's {self.cache.max_seq_len} positions")
         positions = [self.cache.extend(s, 1) for s in slots]
         rows = row_bucket(len(slots))
-        ctx = context_bucket(max(positions) + 1, self.cache.max_seq_len)
-        key = (rows, ctx, sampling.do_sample, float(sampling.temperature), int(sampling.top_k or 0))
-        graph = self._graphs.get(key)
-        if graph is None:
-            for old in [k for k in self._graphs if k[0] == rows and k[2:] == key[2:]]:
+        longest = max(positions) + 1
+        how = (sampling.do_sample, float(sampling.temperature), int(sampling.top_k or 0))
+        fitting = [k for k in self._graphs if k[0] == rows and k[2:] == how and k[1] >= longest]
+        if fitting:
+            graph = self._graphs[min(fitting)]
+        else:
+            for old in [k for k in self._graphs if k[0] == rows and k[2:] == how]:
                 del self._graphs[old]  # a longer context replaces the graph of the shorter one
-            graph = self._graphs[key] = DecodeGraph(self, rows, ctx, sampling)
+            ctx = context_bucket(longest + CONTEXT_HEADROOM, self.cache.max_seq_len)
+            graph = self._graphs[(rows, ctx) + how] = DecodeGraph(self, rows, ctx, sampling)
             graph.capture()
+            self.graph_captures.append((rows, ctx))
         if graph.slots == tuple(slots) and graph.next_tokens == tokens:
             graph.refresh_pages()
         else:

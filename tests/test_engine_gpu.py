@@ -372,35 +372,47 @@ def test_decode_products_that_fuse_the_norms_change_only_rounding(lib, folders, 
         check(fused[:, b], want, "bfloat16")
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_graph_replay_equals_eager_steps(lib, folders, dtype, tmp_path):
-    """Decode through captured graphs gives the tokens of eager steps: across page borders, when the
-    batch shrinks, when the context outgrows the bound a graph was captured for, and with the
-    program's own eager work (prompts of later batches) between the replays."""
+def graph_replay_case(lib, dtype, tmp_path, max_seq_len, prompt_lens, max_tokens):
     from fms_amd.engine import Engine
     from fms_amd.generation import generate_requests
     from fms_amd.sampling import SamplingParams
 
-    kw = dict(CONFIGS["A"], max_expected_seq_len=1400)
+    kw = dict(CONFIGS["A"], max_expected_seq_len=max_seq_len)
     folder = str(tmp_path / "long")
     lib.write_model_folder(folder, lib.LLaMAConfig(**kw), seed=21, std=0.08, norm_std=0.2)
     model = lib.get_model("hf_pretrained", model_path=folder, data_type=dtype)
-    prompts = [tokens_for("A", n, 300 + n) for n in (60, 1000, 3, 64, 129)]
+    prompts = [tokens_for("A", n, 300 + n) for n in prompt_lens]
+    engines = []
     for params in (SamplingParams(do_sample=False), SamplingParams(do_sample=True, temperature=0.9, top_k=20)):
-        eager = Engine(model, max_tokens=2048, max_slots=3, use_graphs=False)
-        graphs = Engine(model, max_tokens=2048, max_slots=3, use_graphs=True)
+        eager = Engine(model, max_tokens=max_tokens, max_slots=3, use_graphs=False)
+        graphs = Engine(model, max_tokens=max_tokens, max_slots=3, use_graphs=True)
         assert graphs.use_graphs
         want = generate_requests(eager, prompts, max_new_tokens=70, sampling=params, seed=9, stop_token_ids=[7])
         got = generate_requests(graphs, prompts, max_new_tokens=70, sampling=params, seed=9, stop_token_ids=[7])
-        if dtype == "float32":
-            assert got == want
-        else:
-            # bfloat16: equal kernels, equal order of operations: equal tokens
-            assert got == want
+        assert got == want  # float32 and bfloat16: equal kernels, equal order of operations: equal tokens
+        captures = len(graphs.graph_captures)
         again = generate_requests(graphs, prompts, max_new_tokens=70, sampling=params, seed=9, stop_token_ids=[7])
-        assert again == got  # the graphs captured above are replayed, not captured anew
+        assert again == got
+        assert len(graphs.graph_captures) == captures  # the graphs captured above are replayed, not captured anew
         graphs.cache.check()
         assert graphs.cache.live_slots() == []
+        engines.append(graphs)
+    return engines
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_replay_equals_eager_steps(lib, folders, dtype, tmp_path):
+    """Decode through captured graphs gives the tokens of eager steps: across page borders, when the
+    batch shrinks, and with the program's own eager work (prompts of later batches) between the replays."""
+    graph_replay_case(lib, dtype, tmp_path, 1400, (60, 1000, 3, 64, 129), 2048)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_graph_for_a_longer_context_replaces_the_shorter_one(lib, folders, dtype, tmp_path):
+    """The second batch of three holds a context beyond the bound (2048) of the graph captured for the first."""
+    for graphs in graph_replay_case(lib, dtype, tmp_path, 4600, (60, 1000, 3, 64, 129, 2100), 4096):
+        captured = graphs.graph_captures
+        assert (4, 2048) in captured and (4, 4096) in captured and captured.index((4, 2048)) < captured.index((4, 4096))
 
 
 # --------------------------------------------------------------------------

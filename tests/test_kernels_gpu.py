@@ -185,7 +185,7 @@ def test_rope_kv_write(ops, dtype, H, K, D, rot):
             assert float(kc[p].abs().sum()) == 0 and float(vc[p].abs().sum()) == 0
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 32])
+@pytest.mark.parametrize("M", [1, 8, 20, 32, 40, 64])
 @pytest.mark.parametrize("H,K,D,rot,E", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 40), (8, 8, 32, 16, 256), (40, 4, 128, 128, 32), (30, 2, 136, 136, 32)])
 def test_qkv_rope_write_equals_the_separate_kernels(ops, M, H, K, D, rot, E):
     """The decode-time fusion (projection + rotation + cache write) against linear followed by rope_kv_write."""
@@ -360,7 +360,7 @@ def test_gated_linear(ops, M, hidden, K):
             torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=4e-2, rtol=2e-2)))
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 17, 32])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 64])
 @pytest.mark.parametrize("N,K,eps", [(48, 24, 1e-5), (96, 176, 1e-6), (4096 + 40, 64, 1e-5), (100, 96, 1e-3), (6144, 32, 1e-5)])
 def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
     """The last product of a branch adds to the float32 stream and leaves the next norm's input; the
