@@ -93,7 +93,6 @@ struct WaveState {
 };
 
 __device__ __forceinline__ bf16x8 load_bf16x8(const bf16* p) { return *reinterpret_cast<const bf16x8*>(p); }
-__device__ __forceinline__ bf16x4 load_bf16x4(const bf16* p) { return *reinterpret_cast<const bf16x4*>(p); }
 
 // One step of the online softmax over 32 keys for the 16*QT query columns of a wave.
 // qreg[qt][c]: this lane's 8 query elements d = c*32 + (lane/16)*8 .. +8 of its column (zero when absent).
@@ -113,6 +112,11 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
   const int g = lane >> 4;
   const int ndt = head_dim / 16;
   const int nchunk = (head_dim + 31) / 32;
+  // Which key sits in which row of the two score tiles is free, as long as the second product pairs every
+  // probability with its value.  Rows are dealt so that lane group g ends up with the probabilities of the
+  // 8 consecutive keys 8 g .. 8 g + 7 (tile a: 8 g + i, tile b: 8 g + 4 + i): their values are then one
+  // 16-byte read per row of the transposed values.
+  const int key_a = (r >> 2) * 8 + (r & 3);
   f32x4 sa[QT], sb[QT];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
@@ -125,8 +129,8 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
       const int d = c * 32 + g * 8;
       bf16x8 ka = {0, 0, 0, 0, 0, 0, 0, 0}, kb = {0, 0, 0, 0, 0, 0, 0, 0};
       if (d < head_dim) {
-        ka = load_bf16x8(kbase + (size_t)r * k_stride + d);
-        kb = load_bf16x8(kbase + (size_t)(16 + r) * k_stride + d);
+        ka = load_bf16x8(kbase + (size_t)key_a * k_stride + d);
+        kb = load_bf16x8(kbase + (size_t)(key_a + 4) * k_stride + d);
       }
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt) {
@@ -149,8 +153,8 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int ja = key0 + g * 4 + i;
-        const int jb = ja + 16;
+        const int ja = key0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
+        const int jb = ja + 4;
         sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale2 : -INFINITY;
         sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale2 : -INFINITY;
         mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
@@ -182,10 +186,7 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
 #pragma unroll
   for (int dt = 0; dt < MAXDT; ++dt) {
     if (dt < ndt) {
-      const bf16* vrow = vbase + (size_t)(dt * 16 + r) * v_stride + g * 4;
-      const bf16x4 va = load_bf16x4(vrow);
-      const bf16x4 vb = load_bf16x4(vrow + 16);
-      const bf16x8 v = {va[0], va[1], va[2], va[3], vb[0], vb[1], vb[2], vb[3]};
+      const bf16x8 v = load_bf16x8(vbase + (size_t)(dt * 16 + r) * v_stride + g * 8);
 #pragma unroll
       for (int qt = 0; qt < QT; ++qt)
         st.acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat[qt], st.acc[qt][dt], 0, 0, 0);
@@ -482,24 +483,25 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
   const int nchunk = (head_dim + 31) / 32;
   const int first = (key0 % PAGE_TOKENS) / 32;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  const bf16x4 zero4 = {0, 0, 0, 0};
+  // Which key sits in which row of the two score tiles is free, as long as the second product pairs every
+  // probability with its value.  Rows are dealt so that lane group g ends up with the probabilities of the
+  // 8 consecutive keys 8 g .. 8 g + 7 (tile a: 8 g + i, tile b: 8 g + 4 + i): their values are then one
+  // 16-byte load per row of the transposed page.
+  const int key_a = (r >> 2) * 8 + (r & 3);
   bf16x8 kreg[HALVES][2][(MAXDT + 1) / 2];
-  bf16x4 vreg[HALVES][MAXDT][2];
+  bf16x8 vreg[HALVES][MAXDT];
 #pragma unroll
   for (int hf = 0; hf < HALVES; ++hf) {
 #pragma unroll
     for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
       const int d = c * 32 + g * 8;
       const bool ok = c < nchunk && d < head_dim;
-      kreg[hf][0][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + r) * head_dim + d) : zero8;
-      kreg[hf][1][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + 16 + r) * head_dim + d) : zero8;
+      kreg[hf][0][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + key_a) * head_dim + d) : zero8;
+      kreg[hf][1][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + key_a + 4) * head_dim + d) : zero8;
     }
 #pragma unroll
-    for (int dt = 0; dt < MAXDT; ++dt) {
-      const bf16* vrow = vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + (first + hf) * 32 + g * 4;
-      vreg[hf][dt][0] = dt < ndt ? load_bf16x4(vrow) : zero4;
-      vreg[hf][dt][1] = dt < ndt ? load_bf16x4(vrow + 16) : zero4;
-    }
+    for (int dt = 0; dt < MAXDT; ++dt)
+      vreg[hf][dt] = dt < ndt ? load_bf16x8(vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + (first + hf) * 32 + g * 8) : zero8;
   }
 #pragma unroll
   for (int hf = 0; hf < HALVES; ++hf) {
@@ -523,8 +525,8 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int ja = k0 + g * 4 + i;
-        const int jb = ja + 16;
+        const int ja = k0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
+        const int jb = ja + 4;
         sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] * scale2 : -INFINITY;
         sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] * scale2 : -INFINITY;
         mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
@@ -547,11 +549,8 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
                          (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
 #pragma unroll
     for (int dt = 0; dt < MAXDT; ++dt) {
-      if (dt < ndt) {
-        const bf16x4 va = vreg[hf][dt][0], vb = vreg[hf][dt][1];
-        const bf16x8 v = {va[0], va[1], va[2], va[3], vb[0], vb[1], vb[2], vb[3]};
-        st.acc[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat, st.acc[0][dt] * alpha, 0, 0, 0);
-      }
+      if (dt < ndt)
+        st.acc[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[hf][dt], pmat, st.acc[0][dt] * alpha, 0, 0, 0);
     }
   }
 }
