@@ -107,4 +107,11 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
   return scratch[16];
 }
 
+// A block-wide barrier that orders LDS traffic only: every wave's LDS writes are done before any wave goes
+// on.  Unlike __syncthreads() it does not wait for global loads in flight, which a kernel that keeps loads
+// of later steps under way while it works on this one must not do.
+__device__ __forceinline__ void block_sync_lds() {
+  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+}
+
 static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -95,21 +95,25 @@ typedef struct {
   float eps;
 } fmsamd_row_scale;
 
-// at most 64 rows: the weights stream once through MFMA registers
+// At most 64 rows: the weights stream once through MFMA registers.  From 17 rows on the product needs a
+// workspace of fmsamd_gemm_skinny_workspace(M, rows of W, K) bytes (slices of K meet there).
+long fmsamd_gemm_skinny_workspace(int M, int rows, int K);
 int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                             int out_dtype, long ldo, int M, int N, int K, const fmsamd_row_scale* row_scale,
-                            hipStream_t stream);
+                            void* workspace, long workspace_bytes, hipStream_t stream);
 int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                   int out_dtype, long ldo, int M, int hidden, int K, int act,
-                                  const fmsamd_row_scale* row_scale, hipStream_t stream);
+                                  const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
+                                  hipStream_t stream);
 // resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, partial_count] = sums
-// of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(N) says;
+// of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(M, N) says;
 // every entry is written).  At most 64 rows.
-int fmsamd_gemm_skinny_residual_partials(int N);
+int fmsamd_gemm_skinny_residual_partials(int M, int N);
 int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                      float* resid, long ldr, const void* norm_w, int norm_w_dtype, void* scaled,
                                      long ldo, float* partials, int partial_count, int M, int N, int K,
-                                     const fmsamd_row_scale* row_scale, hipStream_t stream);
+                                     const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
+                                     hipStream_t stream);
 
 // qkv = x W^T (+ bias) for at most 64 rows with the rotation and the cache write fused into the epilogue;
 // only the query columns of `out` are written
@@ -117,7 +121,8 @@ int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const vo
                                 long ldo, int M, int K, const int* positions, const int* seq_of_token,
                                 const int* block_table, int table_stride, const float* cos_t, const float* sin_t,
                                 int rot_dim, int max_pos, void* k_cache, void* v_cache, int nheads, int kvheads,
-                                int head_dim, const fmsamd_row_scale* row_scale, hipStream_t stream);
+                                int head_dim, const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
+                                hipStream_t stream);
 
 // token choice; rng_state is [rows][2] uint64 (seed, counter), advanced by the kernel
 int fmsamd_sample(const float* logits, long ld, int rows, int vocab, int do_sample, float temperature, int top_k,

@@ -5,12 +5,15 @@
 //     true 32-bit path: no matrix-core shortcut, no reduced-precision inputs.
 //   * gemm_bf16_kernel: bfloat16 in, MFMA 16x16x32 with float32 accumulation,
 //     bfloat16 or float32 out; LDS-tiled 128x128x32.  Any M and N; K % 8 == 0.
-//   * skinny_bf16_kernel: M <= 64 rows of x (decode).  Weight-streaming: a
+//   * skinny_bf16_kernel: M <= 16 rows of x (decode).  Weight-streaming: a
 //     block owns one or two 16-row tiles of W, its waves split K, loads take
 //     long contiguous runs and change to the MFMA layout in LDS, partial
-//     sums meet in LDS.  Optional fused gate: out = act(x Wg^T) * (x Wu^T).
+//     sums meet in LDS.  Epilogues: plain, act(x Wg^T) * (x Wu^T), rotation
+//     and cache write, addition into the residual stream.  The entry points
+//     hand 17 to 64 rows to the kernels of gemm_wide.hip.
 #include "common.h"
 #include "fmsamd.h"
+#include "gemm_epilogue.h"
 
 // ==========================================================================
 // float32
@@ -182,60 +185,8 @@ extern "C" int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const vo
 }
 
 // ==========================================================================
-// bfloat16, M <= 64
+// bfloat16, M <= 16 (and the entry points for M <= 64)
 // ==========================================================================
-
-__device__ __forceinline__ float sk_activate(float x, int kind) {
-  switch (kind) {
-    case FMS_ACT_SILU:
-      return x / (1.f + __expf(-x));
-    case FMS_ACT_GELU:
-      return 0.5f * x * (1.f + erff(x * 0.70710678118654752f));
-    case FMS_ACT_RELU:
-      return fmaxf(x, 0.f);
-    default:
-      return x;
-  }
-}
-
-// What the skinny kernel does with a finished output element.
-#define EPI_PLAIN 0  // store (+ bias)
-#define EPI_GATED 1  // the block's second tile is the "up" half: out = act(first) * second, N is the hidden size
-#define EPI_ROPE 2   // the output row is [queries | keys | values] of attention: rotate q and k, store q, and
-                     // write k and v into their cache pages (layout: see rope.hip)
-#define EPI_RESID 3  // add the product to the float32 residual stream in place, store the new stream times the
-                     // next norm's weight in the activation type, and leave the rows' sums of squares by tile
-
-// The rows of x are not yet divided by their root mean square: the kernel that made them left, for each
-// row, `count` partial sums of squares (partials[m * count + i]).  The product is multiplied by
-// rsqrt(sum / width + eps) of its row before the bias.  partials == null: the rows are taken as they are.
-struct RowScale {
-  const float* partials;
-  int count;
-  float inv_width, eps;
-};
-
-struct ResidEpilogue {
-  float* resid;  // [M, N] float32, read and written
-  long ldr;
-  const void* norm_w;  // [N] or null
-  int norm_w_f32;
-  float* partials;  // [M, tiles]: sum over the tile's 16 columns of the new stream squared
-  int tiles;
-};
-
-struct RopeEpilogue {
-  const int* positions;     // [M]
-  const int* seq_of_token;  // [M], -1: padding row
-  const int* block_table;
-  int table_stride;
-  const float* cos_t;  // [max_pos, rot_dim/2] or null
-  const float* sin_t;
-  int rot_dim, max_pos;
-  bf16* k_cache;  // null: queries only
-  bf16* v_cache;
-  int nheads, kvheads, head_dim;
-};
 
 // NTB: 16-row tiles of W per block (the second tile starts `tile2_offset` rows after the first).
 // MT : 16-row tiles of x.
@@ -573,7 +524,8 @@ static int row_scale_of(const fmsamd_row_scale* in, int K, RowScale* out) {
 // out[M, N] = x[M, K] w[N, K]^T (+ bias).  M <= 64.
 extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                        void* out, int out_dtype, long ldo, int M, int N, int K,
-                                       const fmsamd_row_scale* row_scale, hipStream_t stream) {
+                                       const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
+                                       hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
@@ -581,15 +533,16 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N, "gemm_skinny_bf16: leading dimensions too small");
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_bf16: unknown output dtype %d", out_dtype);
-  const int mt = ceil_div(M, 16);
+  if (M > 16)
+    return wide_product(EPI_PLAIN, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, scale, RopeEpilogue{},
+                        ResidEpilogue{}, workspace, workspace_bytes, stream);
   const int rows = skinny_rows_per_block(N);
 #define FMS_LS(NTB, MT) \
   launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, rows, stream, scale)
-  if (rows > 16) {
-    if (mt == 1) FMS_LS(2, 1); else if (mt == 2) FMS_LS(2, 2); else if (mt == 3) FMS_LS(2, 3); else FMS_LS(2, 4);
-  } else {
-    if (mt == 1) FMS_LS(1, 1); else if (mt == 2) FMS_LS(1, 2); else if (mt == 3) FMS_LS(1, 3); else FMS_LS(1, 4);
-  }
+  if (rows > 16)
+    FMS_LS(2, 1);
+  else
+    FMS_LS(1, 1);
 #undef FMS_LS
   FMS_LAUNCH_CHECK("gemm_skinny_bf16");
   return 0;
@@ -598,7 +551,8 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
 // out[M, hidden] = act(x Wg^T + bg) * (x Wu^T + bu) with w = [Wg; Wu] stacked, [2*hidden, K].  M <= 64.
 extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias,
                                              int bias_dtype, void* out, int out_dtype, long ldo, int M, int hidden,
-                                             int K, int act, const fmsamd_row_scale* row_scale, hipStream_t stream) {
+                                             int K, int act, const fmsamd_row_scale* row_scale, void* workspace,
+                                             long workspace_bytes, hipStream_t stream) {
   if (M == 0 || hidden == 0) return 0;
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
@@ -609,11 +563,13 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
   FMS_REQUIRE(ldx >= K && ldo >= hidden, "gemm_skinny_gated_bf16: leading dimensions too small");
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_gated_bf16: unknown output dtype %d", out_dtype);
   FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gemm_skinny_gated_bf16: unknown activation %d", act);
-  const int mt = ceil_div(M, 16);
+  if (M > 16)
+    return wide_product(EPI_GATED, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, scale,
+                        RopeEpilogue{}, ResidEpilogue{}, workspace, workspace_bytes, stream);
 #define FMS_LG(MT) \
   launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, 16, \
                                   stream, scale)
-  if (mt == 1) FMS_LG(1); else if (mt == 2) FMS_LG(2); else if (mt == 3) FMS_LG(3); else FMS_LG(4);
+  FMS_LG(1);
 #undef FMS_LG
   FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
   return 0;
@@ -627,7 +583,8 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
                                            const int* seq_of_token, const int* block_table, int table_stride,
                                            const float* cos_t, const float* sin_t, int rot_dim, int max_pos,
                                            void* k_cache, void* v_cache, int nheads, int kvheads, int head_dim,
-                                           const fmsamd_row_scale* row_scale, hipStream_t stream) {
+                                           const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
+                                           hipStream_t stream) {
   if (M == 0) return 0;
   const int N = (nheads + 2 * kvheads) * head_dim;
   RowScale scale;
@@ -644,15 +601,16 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   FMS_REQUIRE(cos_t == nullptr || (max_pos > 0 && sin_t != nullptr), "qkv_rope_skinny_bf16: empty rotary table");
   RopeEpilogue rope{positions, seq_of_token, block_table, table_stride, rot_dim > 0 ? cos_t : nullptr, sin_t, rot_dim,
                     max_pos, (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim};
+  if (M > 16)
+    return wide_product(EPI_ROPE, x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, scale, rope,
+                        ResidEpilogue{}, workspace, workspace_bytes, stream);
   const int rows = skinny_rows_per_block(N);
-  const int mt = ceil_div(M, 16);
 #define FMS_LR(NTB, MT) \
   launch_skinny<NTB, MT, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
-  if (rows > 16) {
-    if (mt == 1) FMS_LR(2, 1); else if (mt == 2) FMS_LR(2, 2); else if (mt == 3) FMS_LR(2, 3); else FMS_LR(2, 4);
-  } else {
-    if (mt == 1) FMS_LR(1, 1); else if (mt == 2) FMS_LR(1, 2); else if (mt == 3) FMS_LR(1, 3); else FMS_LR(1, 4);
-  }
+  if (rows > 16)
+    FMS_LR(2, 1);
+  else
+    FMS_LR(1, 1);
 #undef FMS_LR
   FMS_LAUNCH_CHECK("qkv_rope_skinny_bf16");
   return 0;
@@ -666,16 +624,23 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
 //                    [M, partial_count], partial_count >= fmsamd_gemm_skinny_residual_partials(N)
 // A product that takes `scaled` with these partials as its deferred row norm then equals the product of the
 // normed stream.  M <= 64.
-extern "C" int fmsamd_gemm_skinny_residual_partials(int N) {
+extern "C" int fmsamd_gemm_skinny_residual_partials(int M, int N) {
+  if (M > 16) return ceil_div(N, 16);
   const int rows = skinny_rows_per_block(N);
   return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
+}
+
+// Bytes of workspace that the products for at most 64 rows need (none up to 16 rows).  rows: all rows of W.
+extern "C" long fmsamd_gemm_skinny_workspace(int M, int rows, int K) {
+  return M > 16 && M <= 64 ? wide_workspace_bytes(M, rows, K) : 0;
 }
 
 extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias,
                                                 int bias_dtype, float* resid, long ldr, const void* norm_w,
                                                 int norm_w_dtype, void* scaled, long ldo, float* partials,
                                                 int partial_count, int M, int N, int K,
-                                                const fmsamd_row_scale* row_scale, hipStream_t stream) {
+                                                const fmsamd_row_scale* row_scale, void* workspace,
+                                                long workspace_bytes, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
   FMS_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 64)", M, N, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_residual_bf16: K=%d and the row stride %ld must be multiples of 8",
@@ -687,19 +652,24 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
   const int rows = skinny_rows_per_block(N);
-  const int tiles = ceil_div(N, rows) * (rows > 16 ? 2 : 1);
+  const int tiles = fmsamd_gemm_skinny_residual_partials(M, N);
   FMS_REQUIRE(partial_count >= tiles, "gemm_skinny_residual_bf16: room for %d partial sums per row, %d needed",
               partial_count, tiles);
   ResidEpilogue res{resid, ldr, norm_w, norm_w_dtype == FMS_F32, partials, partial_count};
-  const int mt = ceil_div(M, 16);
+  if (M > 16) {
+    res.tiles = tiles;  // the finish kernel writes exactly these
+    FMS_REQUIRE(partial_count == tiles, "gemm_skinny_residual_bf16: %d partial sums per row, %d expected", partial_count,
+                tiles);
+    return wide_product(EPI_RESID, x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, scale,
+                        RopeEpilogue{}, res, workspace, workspace_bytes, stream);
+  }
 #define FMS_LX(NTB, MT)                                                                                              \
   launch_skinny<NTB, MT, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, \
                                     scale, RopeEpilogue{}, res)
-  if (rows > 16) {
-    if (mt == 1) FMS_LX(2, 1); else if (mt == 2) FMS_LX(2, 2); else if (mt == 3) FMS_LX(2, 3); else FMS_LX(2, 4);
-  } else {
-    if (mt == 1) FMS_LX(1, 1); else if (mt == 2) FMS_LX(1, 2); else if (mt == 3) FMS_LX(1, 3); else FMS_LX(1, 4);
-  }
+  if (rows > 16)
+    FMS_LX(2, 1);
+  else
+    FMS_LX(1, 1);
 #undef FMS_LX
   FMS_LAUNCH_CHECK("gemm_skinny_residual_bf16");
   return 0;

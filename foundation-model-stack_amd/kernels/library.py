@@ -36,13 +36,14 @@ _SIGNATURES = {
     "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, P],
-    "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P],
+    "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
     "fmsamd_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
-    "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P, P],
-    "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P, P],
-    "fmsamd_gemm_skinny_residual_partials": [I],
-    "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P],
+    "fmsamd_gemm_skinny_workspace": [I, I, I],
+    "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P, P, L, P],
+    "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P, P, L, P],
+    "fmsamd_gemm_skinny_residual_partials": [I, I],
+    "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P, L, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
 }
@@ -85,6 +86,7 @@ def load(verbose: bool = True) -> ctypes.CDLL:
         lib.fmsamd_argmax_workspace.restype = c_long
         lib.fmsamd_argmax_workspace.argtypes = [I, I]
         lib.fmsamd_attn_decode_workspace.restype = c_long
+        lib.fmsamd_gemm_skinny_workspace.restype = c_long
         lib.fmsamd_attn_decode_workspace.argtypes = [I, I, I, I]
         lib.path = path
         _lib = lib

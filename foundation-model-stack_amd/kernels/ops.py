@@ -196,6 +196,15 @@ class RowNorm:
         self.partials, self.eps = partials, float(eps)
 
 
+def _skinny_workspace(rows: int, weight_rows: int, K: int, device):
+    """(pointer, bytes) of the workspace a product for `rows` rows of x needs; (None, 0) up to 16 rows."""
+    n = load().fmsamd_gemm_skinny_workspace(rows, weight_rows, K)
+    if n <= 0:
+        return None, 0
+    ws = torch.empty(n // 4, dtype=torch.float32, device=device)
+    return ws, n
+
+
 class _RowScaleArg(ctypes.Structure):
     _fields_ = [("partials", ctypes.c_void_p), ("count", ctypes.c_int), ("eps", ctypes.c_float)]
 
@@ -251,11 +260,12 @@ def qkv_rope_write(
     if k_cache is not None:
         _check_cache(k_cache, v_cache, kvheads, head_dim, torch.bfloat16)
     out = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
+    ws, ws_bytes = _skinny_workspace(M, N, K, x.device)
     check(load().fmsamd_qkv_rope_skinny_bf16(
         x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
         out.data_ptr(), out.stride(0), M, K, positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
         block_table.stride(0), _ptr(cos), _ptr(sin), rot_dim if cos is not None else 0, max_pos, _ptr(k_cache),
-        _ptr(v_cache), nheads, kvheads, head_dim, _row_scale(row_norm, M), _stream()))
+        _ptr(v_cache), nheads, kvheads, head_dim, _row_scale(row_norm, M), _ptr(ws), ws_bytes, _stream()))
     return out
 
 
@@ -453,8 +463,10 @@ def linear(
     bcode = _code(bias.dtype) if bias is not None else 0
     if M <= SKINNY_FAST_ROWS or (M <= SKINNY_MAX_ROWS and not (allow_library and out_dtype == torch.bfloat16)):
         out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+        ws, ws_bytes = _skinny_workspace(M, N, K, x.device)
         check(lib.fmsamd_gemm_skinny_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), bcode, out.data_ptr(),
-                                          _code(out_dtype), out.stride(0), M, N, K, _row_scale(row_norm, M), _stream()))
+                                          _code(out_dtype), out.stride(0), M, N, K, _row_scale(row_norm, M), _ptr(ws),
+                                          ws_bytes, _stream()))
         return out
     if allow_library and out_dtype == torch.bfloat16:
         out = torch.matmul(x, weight.t())  # vendor library GEMM, float32 accumulation
@@ -498,12 +510,13 @@ def linear_into_stream(
         raise ValueError(f"the norm weight is a contiguous float32 or bfloat16 [{N}] tensor")
     scaled = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
     lib = load()
-    partials = torch.empty(M, lib.fmsamd_gemm_skinny_residual_partials(N), dtype=torch.float32, device=x.device)
+    partials = torch.empty(M, lib.fmsamd_gemm_skinny_residual_partials(M, N), dtype=torch.float32, device=x.device)
+    ws, ws_bytes = _skinny_workspace(M, N, K, x.device)
     check(lib.fmsamd_gemm_skinny_residual_bf16(
         x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
         resid.data_ptr(), resid.stride(0), _ptr(norm_weight), _code(norm_weight.dtype) if norm_weight is not None else 0,
         scaled.data_ptr(), scaled.stride(0), partials.data_ptr(), partials.shape[1], M, N, K, _row_scale(row_norm, M),
-        _stream()))
+        _ptr(ws), ws_bytes, _stream()))
     return scaled, RowNorm(partials, eps)
 
 
@@ -527,10 +540,11 @@ def gated_linear(
         if bias is not None and (bias.shape != (2 * hidden,) or not bias.is_contiguous()):
             raise ValueError(f"bias must be a contiguous [{2 * hidden}] tensor")
         out = torch.empty(M, hidden, dtype=torch.bfloat16, device=x.device)
+        ws, ws_bytes = _skinny_workspace(M, 2 * hidden, K, x.device)
         check(load().fmsamd_gemm_skinny_gated_bf16(x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias),
                                                    _code(bias.dtype) if bias is not None else 0, out.data_ptr(), BF16,
                                                    out.stride(0), M, hidden, K, ACTIVATIONS[activation],
-                                                   _row_scale(row_norm, M), _stream()))
+                                                   _row_scale(row_norm, M), _ptr(ws), ws_bytes, _stream()))
         return out
     if row_norm is not None:
         raise ValueError("a deferred row norm goes with the bfloat16 product of at most 64 rows")
