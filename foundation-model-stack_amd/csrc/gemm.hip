@@ -194,7 +194,7 @@ extern "C" int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const vo
 // UNR: groups of 128 k-values whose loads a wave issues before it multiplies: what keeps enough
 // bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 4 loads of 16 bytes outstanding).
 template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typename BiasT>
-__global__ void __launch_bounds__(SK_WAVES* WAVE)
+__global__ void __launch_bounds__(SK_WAVES* WAVE) __attribute__((amdgpu_waves_per_eu(4)))  // two blocks a compute unit
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
                        int rows_per_block, RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
@@ -226,9 +226,11 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
   }
 
   // Loads whose data the epilogue needs are issued here, ahead of the weight stream, so that their latency
-  // is not paid at the end: the first partial sums of a deferred row norm (a wave per row, four rows and
-  // 256 sums deep) and the residual stream with the next norm's weight.
-  constexpr int PRE_ROWS = 4, PRE_DEPTH = 4;
+  // is not paid at the end: the first partial sums of a deferred row norm (a wave per row, 256 sums deep) and the residual stream with the next norm's weight.
+  // None of these loads sits behind a branch, and none of their data is touched before the epilogue: either
+  // would make the compiler wait for the load on the spot.  What is out of range is read from a valid address
+  // and set aside when it is used.
+  constexpr int PRE_ROWS = (MT * 16 + SK_WAVES - 1) / SK_WAVES, PRE_DEPTH = 4;  // every row of x, 256 sums deep
   float pre[PRE_ROWS][PRE_DEPTH];
   if (scale.partials != nullptr) {
 #pragma unroll
@@ -236,12 +238,13 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 #pragma unroll
       for (int j = 0; j < PRE_DEPTH; ++j) {
         const int m = wave + i * SK_WAVES, b = lane + j * WAVE;
-        pre[i][j] = (m < M && b < scale.count) ? scale.partials[(size_t)m * scale.count + b] : 0.f;
+        pre[i][j] = scale.partials[(size_t)(m < M ? m : 0) * scale.count + (b < scale.count ? b : 0)];
       }
   }
   constexpr int OUT_TILES = GATED ? 1 : NTB;
   constexpr int ROUNDS = (OUT_TILES * MT * 256 + SK_WAVES * WAVE - 1) / (SK_WAVES * WAVE);
   float pre_resid[ROUNDS], pre_nw[ROUNDS];  // EPI_ROPE: cosine and sine of the element's angle
+  bf16 pre_nw16[ROUNDS];
   if (EPI == EPI_ROPE) {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
@@ -250,12 +253,13 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       const int n = n0 + ((idx >> 8) / MT) * 16 + (idx & 15);
       const int hh = n / rope.head_dim, d = n - hh * rope.head_dim;
       pre_resid[rd] = 1.f, pre_nw[rd] = 0.f;
-      if (idx < OUT_TILES * MT * 256 && m < M && n < n_end && hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr &&
-          d < rope.rot_dim) {
-        const int pos = rope.positions[m];
-        const int tpos = pos < rope.max_pos ? pos : rope.max_pos - 1;  // the host has checked the range
-        pre_resid[rd] = rope.cos_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
-        pre_nw[rd] = rope.sin_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
+      if (rope.cos_t != nullptr) {  // uniform
+        const bool rotates = m < M && n < n_end && hh < rope.nheads + rope.kvheads && d < rope.rot_dim;
+        const int pos = rope.positions[m < M ? m : 0];
+        const int tpos = pos < 0 ? 0 : (pos < rope.max_pos ? pos : rope.max_pos - 1);  // the host has checked the range
+        const size_t at = rotates ? (size_t)tpos * (rope.rot_dim / 2) + d / 2 : 0;
+        pre_resid[rd] = rope.cos_t[at];
+        pre_nw[rd] = rope.sin_t[at];
       }
     }
   }
@@ -266,10 +270,15 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       const int m = ((idx >> 8) % MT) * 16 + ((idx >> 4) & 15);
       const int n = n0 + ((idx >> 8) / MT) * 16 + (idx & 15);
       const bool live = idx < OUT_TILES * MT * 256 && m < M && n < n_end;
-      pre_resid[rd] = live ? res.resid[(size_t)m * res.ldr + n] : 0.f;
+      pre_resid[rd] = res.resid[live ? (size_t)m * res.ldr + n : 0];
       pre_nw[rd] = 1.f;
-      if (live && res.norm_w != nullptr)
-        pre_nw[rd] = res.norm_w_f32 ? ((const float*)res.norm_w)[n] : to_f32(((const bf16*)res.norm_w)[n]);
+      pre_nw16[rd] = (bf16)1.f;
+      if (res.norm_w != nullptr) {  // uniform
+        if (res.norm_w_f32)
+          pre_nw[rd] = ((const float*)res.norm_w)[live ? n : 0];
+        else
+          pre_nw16[rd] = ((const bf16*)res.norm_w)[live ? n : 0];
+      }
     }
   }
 
@@ -305,10 +314,11 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
         const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : n_end;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
+          // a row past the block's last is read from the block's first (its sums are never stored), a piece
+          // past K from the row's start (it meets zeros of x)
           const int n = nbase + 4 * q + lrow;
-          wreg[u][t][q] = (kok && n < limit)
-                              ? __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w + (size_t)n * K + k))
-                              : zero;
+          const size_t at = (size_t)(n < limit ? n : nbase) * K + (kok ? k : 0);
+          wreg[u][t][q] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w + at));
         }
       }
 #pragma unroll
@@ -317,7 +327,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
         for (int q = 0; q < 4; ++q) {
           const int m = t * 16 + 4 * q + lrow;
           if (t * 16 + 4 * q < M)  // uniform: whole instructions fall away for few rows
-            xreg[u][t][q] = (kok && m < M) ? *reinterpret_cast<const bf16x8*>(x + (size_t)m * ldx + k) : zero;
+            xreg[u][t][q] = *reinterpret_cast<const bf16x8*>(x + (size_t)(m < M ? m : 0) * ldx + (kok ? k : 0));
         }
     }
 #pragma unroll
@@ -347,7 +357,8 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
           const int row = 4 * q + lrow;
           const bool loaded = j * 16 + 4 * q < M;  // uniform
           if (MT == 1 && !loaded) continue;        // one tile only: its empty rows were zeroed at the start
-          *reinterpret_cast<bf16x8*>(stage_x + row * 128 + ((seg ^ row) & 15) * 8) = loaded ? xreg[u][j][q] : zero;
+          const bool inside = loaded && j * 16 + row < M && (c0 + u) * 128 + seg * 8 < K;
+          *reinterpret_cast<bf16x8*>(stage_x + row * 128 + ((seg ^ row) & 15) * 8) = inside ? xreg[u][j][q] : zero;
         }
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
@@ -380,7 +391,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       if (m < M) {
         float sum = 0.f;
 #pragma unroll
-        for (int j = 0; j < PRE_DEPTH; ++j) sum += pre[i][j];
+        for (int j = 0; j < PRE_DEPTH; ++j) sum += lane + j * WAVE < scale.count ? pre[i][j] : 0.f;
         for (int b = lane + PRE_DEPTH * WAVE; b < scale.count; b += WAVE) sum += scale.partials[(size_t)m * scale.count + b];
         sum = wave_sum(sum);
         if (lane == 0) s_scale[m] = rsqrtf(sum * scale.inv_width + scale.eps);
@@ -432,8 +443,8 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       const int D = rope.head_dim;
       const int hh = n / D, d = n - hh * D;
       const int pos = s_pos[m], seq = s_seq[m];
-      {
-        const float c = pre_resid[rd], sn = pre_nw[rd];  // 1 and 0 where nothing rotates
+      if (rope.cos_t != nullptr && hh < rope.nheads + rope.kvheads && d < rope.rot_dim) {
+        const float c = pre_resid[rd], sn = pre_nw[rd];
         v = (d & 1) ? sn * partner + c * v : c * v - sn * partner;
       }
       if (hh < rope.nheads) {
@@ -455,7 +466,8 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
         if (bias) v += to_f32(bias[n]);
         stream = pre_resid[rd] + v;
         res.resid[(size_t)m * res.ldr + n] = stream;
-        out[(size_t)m * ldo + n] = from_f32<OutT>(stream * pre_nw[rd]);
+        const float nw = (res.norm_w != nullptr && !res.norm_w_f32) ? to_f32(pre_nw16[rd]) : pre_nw[rd];
+        out[(size_t)m * ldo + n] = from_f32<OutT>(stream * nw);
       }
       // the 16 columns of a tile sit in 16 neighbouring lanes
       float sq = stream * stream;
