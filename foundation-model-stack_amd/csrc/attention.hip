@@ -471,38 +471,16 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 // of a page (keys and values) are issued together before any arithmetic.
 // Splits of one token meet in attn_decode_merge_kernel.
 // ==========================================================================
+// The arithmetic of HALVES halves of 32 keys starting at key0, for operands that are already in registers:
+// kreg[hf][tile][c] the keys of the two score tiles (rows dealt as key_a below says), vreg[hf][dt] the values.
 template <int MAXDT, int HALVES>
-__device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
-                                            int qlo, int key0, const bf16* __restrict__ kp,
-                                            const bf16* __restrict__ vp, int head_dim, float scale2) {
-  // HALVES halves of 32 keys starting at key0 (kp/vp point at the page, `first` is the half inside it)
+__device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
+                                            int qlo, int key0, const bf16x8 (&kreg)[HALVES][2][(MAXDT + 1) / 2],
+                                            const bf16x8 (&vreg)[HALVES][MAXDT], int head_dim, float scale2) {
   const int lane = threadIdx.x & (WAVE - 1);
-  const int r = lane & 15;
   const int g = lane >> 4;
   const int ndt = head_dim / 16;
   const int nchunk = (head_dim + 31) / 32;
-  const int first = (key0 % PAGE_TOKENS) / 32;
-  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-  // Which key sits in which row of the two score tiles is free, as long as the second product pairs every
-  // probability with its value.  Rows are dealt so that lane group g ends up with the probabilities of the
-  // 8 consecutive keys 8 g .. 8 g + 7 (tile a: 8 g + i, tile b: 8 g + 4 + i): their values are then one
-  // 16-byte load per row of the transposed page.
-  const int key_a = (r >> 2) * 8 + (r & 3);
-  bf16x8 kreg[HALVES][2][(MAXDT + 1) / 2];
-  bf16x8 vreg[HALVES][MAXDT];
-#pragma unroll
-  for (int hf = 0; hf < HALVES; ++hf) {
-#pragma unroll
-    for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
-      const int d = c * 32 + g * 8;
-      const bool ok = c < nchunk && d < head_dim;
-      kreg[hf][0][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + key_a) * head_dim + d) : zero8;
-      kreg[hf][1][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + key_a + 4) * head_dim + d) : zero8;
-    }
-#pragma unroll
-    for (int dt = 0; dt < MAXDT; ++dt)
-      vreg[hf][dt] = dt < ndt ? load_bf16x8(vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + (first + hf) * 32 + g * 8) : zero8;
-  }
 #pragma unroll
   for (int hf = 0; hf < HALVES; ++hf) {
     const int k0 = key0 + hf * 32;
@@ -555,6 +533,100 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
   }
 }
 
+template <int MAXDT, int HALVES>
+__device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x8 (&qreg)[(MAXDT + 1) / 2], int qpos,
+                                            int qlo, int key0, const bf16* __restrict__ kp,
+                                            const bf16* __restrict__ vp, int head_dim, float scale2) {
+  // HALVES halves of 32 keys starting at key0 (kp/vp point at the page, `first` is the half inside it)
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int ndt = head_dim / 16;
+  const int nchunk = (head_dim + 31) / 32;
+  const int first = (key0 % PAGE_TOKENS) / 32;
+  const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  // Which key sits in which row of the two score tiles is free, as long as the second product pairs every
+  // probability with its value.  Rows are dealt so that lane group g ends up with the probabilities of the
+  // 8 consecutive keys 8 g .. 8 g + 7 (tile a: 8 g + i, tile b: 8 g + 4 + i): their values are then one
+  // 16-byte load per row of the transposed page.
+  const int key_a = (r >> 2) * 8 + (r & 3);
+  bf16x8 kreg[HALVES][2][(MAXDT + 1) / 2];
+  bf16x8 vreg[HALVES][MAXDT];
+#pragma unroll
+  for (int hf = 0; hf < HALVES; ++hf) {
+#pragma unroll
+    for (int c = 0; c < (MAXDT + 1) / 2; ++c) {
+      const int d = c * 32 + g * 8;
+      const bool ok = c < nchunk && d < head_dim;
+      kreg[hf][0][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + key_a) * head_dim + d) : zero8;
+      kreg[hf][1][c] = ok ? load_bf16x8(kp + (size_t)((first + hf) * 32 + key_a + 4) * head_dim + d) : zero8;
+    }
+#pragma unroll
+    for (int dt = 0; dt < MAXDT; ++dt)
+      vreg[hf][dt] = dt < ndt ? load_bf16x8(vp + (size_t)(dt * 16 + r) * PAGE_TOKENS + (first + hf) * 32 + g * 8) : zero8;
+  }
+  decode_math<MAXDT, HALVES>(st, qreg, qpos, qlo, key0, kreg, vreg, head_dim, scale2);
+}
+
+// A whole page of head size 128 by way of the wave's own 16 KB of LDS.  The page of a kv head is 16 KB of
+// keys and 16 KB of values, each contiguous: the wave loads them 1 KB an instruction (what the memory system
+// streams best; the operand layout takes 64 bytes from each of 16 rows and fetches every line twice), writes
+// them to LDS as loaded and reads the MFMA operands back: first the keys, then, through the same buffer, the
+// values.  16-byte pieces are XOR-swizzled so that both directions spread over the banks.
+__device__ __forceinline__ void decode_page_staged(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
+                                                   int key0, const bf16* __restrict__ kp, const bf16* __restrict__ vp,
+                                                   bf16* __restrict__ buf, float scale2) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  bf16x8 kraw[16], vraw[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) kraw[i] = load_bf16x8(kp + i * 512 + lane * 8);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) vraw[i] = load_bf16x8(vp + i * 512 + lane * 8);
+
+  // keys: row = token (256 bytes = 16 pieces), piece ^ key(token); the 16 tokens of a score tile have the keys 0..15
+  {
+    const int piece = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int token = i * 4 + (lane >> 4);
+      const int key = (((token >> 3) & 3) << 2) | (token & 3);
+      *reinterpret_cast<bf16x8*>(buf + token * 128 + ((piece ^ key) & 15) * 8) = kraw[i];
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  bf16x8 kreg[2][2][4], vreg[2][8];
+  const int key_a = (r >> 2) * 8 + (r & 3);  // its swizzle key is r, and so is that of key_a + 4
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int tile = 0; tile < 2; ++tile)
+#pragma unroll
+      for (int c = 0; c < 4; ++c)
+        kreg[hf][tile][c] = *reinterpret_cast<const bf16x8*>(buf + (hf * 32 + key_a + 4 * tile) * 128 + (((c * 4 + g) ^ r) & 15) * 8);
+  __builtin_amdgcn_wave_barrier();
+  // values: row = d (128 bytes = 8 pieces of 8 tokens), piece ^ (d / 2): two rows fill the banks once
+  {
+    const int piece = lane & 7;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int d = i * 8 + (lane >> 3);
+      *reinterpret_cast<bf16x8*>(buf + d * 64 + ((piece ^ (d >> 1)) & 7) * 8) = vraw[i];
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) {
+      const int d = dt * 16 + r;
+      vreg[hf][dt] = *reinterpret_cast<const bf16x8*>(buf + d * 64 + (((hf * 4 + g) ^ (d >> 1)) & 7) * 8);
+    }
+  __builtin_amdgcn_wave_barrier();
+  decode_math<8, 2>(st, qreg, qpos, qlo, key0, kreg, vreg, 128, scale2);
+}
+
 // The pages that split `split` of `n_splits` takes of a sequence whose visible keys are lo..pos: every
 // sequence's own pages are dealt out evenly, so that in a batch of unequal lengths every block has work in
 // proportion to its sequence.  Returns the number of splits that have pages at all (the first ones).
@@ -571,15 +643,20 @@ __device__ __forceinline__ int split_pages(int lo, int pos, int n_splits, int sp
 // meet in LDS; the splits of a token meet in the merge kernel.  (Merging in the block that finishes last,
 // behind a device-wide fence and a counter, was measured four times slower: the fence writes back and
 // invalidates the whole L2 of the block's XCD while the other blocks stream through it.)
-template <int MAXDT, int MAXW>
-__global__ void __launch_bounds__(MAXW* WAVE)
+// STAGED (head size 128 only): pages go through LDS (decode_page_staged), 16 KB a wave.
+template <int MAXDT, int MAXW, bool STAGED>
+__global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu(MAXDT <= 8 ? 2 : 1)))
     attn_decode_bf16_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                             float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
                             int window, int tile_cols) {
-  extern __shared__ float lds[];  // [wave][tile_cols columns][head_dim + 2]
+  extern __shared__ float lds_dynamic[];  // not staged: [wave][tile_cols columns][head_dim + 2]
+  __shared__ __attribute__((aligned(16))) bf16 stage[STAGED ? MAXW * 8192 : 8];
+  // where the waves' partial results meet: a region of its own, or (staged) the head of each wave's page buffer
+  float* const lds = STAGED ? reinterpret_cast<float*>(stage) : lds_dynamic;
+  const int wave_stride = STAGED ? 4096 : tile_cols * (head_dim + 2);  // floats
   const int split = blockIdx.x;
   const int group = nheads / kvheads;
   const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
@@ -617,7 +694,10 @@ __global__ void __launch_bounds__(MAXW* WAVE)
     const size_t phys = (size_t)bt[pi];
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
-    if (MAXDT <= 8) {
+    if (STAGED) {
+      if constexpr (MAXDT == 8)
+        decode_page_staged(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, stage + wave * 8192, scale * LOG2E);
+    } else if (MAXDT <= 8) {
       decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
     } else {  // large heads: half a page at a time keeps the loads in registers
       decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
@@ -632,7 +712,7 @@ __global__ void __launch_bounds__(MAXW* WAVE)
   l += __shfl_xor(l, 16, WAVE);
   l += __shfl_xor(l, 32, WAVE);
   if (r < cols) {
-    float* dst = lds + ((size_t)wave * tile_cols + r) * cstride;
+    float* dst = lds + (size_t)wave * wave_stride + r * cstride;
     if (g == 0) {
       dst[head_dim] = st.m[0];
       dst[head_dim + 1] = l;
@@ -648,10 +728,10 @@ __global__ void __launch_bounds__(MAXW* WAVE)
     const int c = idx / head_dim;
     const int d = idx % head_dim;
     float m = -1e30f;
-    for (int w = 0; w < n_waves; ++w) m = fmaxf(m, lds[((size_t)w * tile_cols + c) * cstride + head_dim]);
+    for (int w = 0; w < n_waves; ++w) m = fmaxf(m, lds[(size_t)w * wave_stride + c * cstride + head_dim]);
     float o = 0.f, lsum = 0.f;
     for (int w = 0; w < n_waves; ++w) {
-      const float* src = lds + ((size_t)w * tile_cols + c) * cstride;
+      const float* src = lds + (size_t)w * wave_stride + c * cstride;
       const float f = __builtin_amdgcn_exp2f(src[head_dim] - m);  // maxima are base-2 logarithms
       o += f * src[d];
       lsum += f * src[head_dim + 1];
@@ -805,7 +885,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        const int* block_table, int table_stride, const void* k_cache,
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
                                        float scale, int window, int max_context, int pages_per_split, int waves,
-                                       hipStream_t stream) {
+                                       int staged, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
@@ -828,17 +908,24 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   float* part_o = (float*)workspace;
   float* part_ml = part_o ? part_o + (size_t)n_tokens * nheads * n_splits * head_dim : nullptr;
   dim3 grid(n_splits, kvheads * tiles_per_kv, n_tokens);
-#define FMS_DC(M, MAXW)                                                                                              \
-  attn_decode_bf16_kernel<M, MAXW><<<grid, dim3(waves * WAVE), lds_bytes, stream>>>(                                 \
+#define FMS_DC(M, MAXW, STAGED, LDS)                                                                                 \
+  attn_decode_bf16_kernel<M, MAXW, STAGED><<<grid, dim3(waves * WAVE), LDS, stream>>>(                               \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
       window, tile_cols)
-  if (head_dim <= 64)
-    FMS_DC(4, 8);
+  FMS_REQUIRE(staged == 0 || head_dim == 128, "attn_decode_bf16: pages go through LDS for head size 128 only");
+  if (staged != 0) {
+    // the waves' results meet in the page buffers: 16 KB a wave hold 16 columns of 130 floats
+    if (waves <= 4)
+      FMS_DC(8, 4, true, 0);
+    else
+      FMS_DC(8, 8, true, 0);
+  } else if (head_dim <= 64)
+    FMS_DC(4, 8, false, lds_bytes);
   else if (head_dim <= 128)
-    FMS_DC(8, 8);
+    FMS_DC(8, 8, false, lds_bytes);
   else
-    FMS_DC(16, 4);  // large heads need the registers of a smaller block
+    FMS_DC(16, 4, false, lds_bytes);  // large heads need the registers of a smaller block
 #undef FMS_DC
   FMS_LAUNCH_CHECK("attn_decode_bf16");
   if (n_splits > 1) {

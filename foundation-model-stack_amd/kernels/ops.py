@@ -333,6 +333,7 @@ def attention(
     pages_per_block: int = 0,
     waves: int = 0,
     force_generic: bool = False,
+    staged: Optional[bool] = None,
 ) -> torch.Tensor:
     """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim].
 
@@ -370,7 +371,8 @@ def attention(
         check(lib.fmsamd_attn_decode_bf16(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _ptr(ws), ws_bytes,
                                           positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), T, nheads, kvheads,
-                                          head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves), _stream()))
+                                          head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves),
+                                          int(bool(staged)) if staged is not None else int(head_dim == 128), _stream()))
         return out
     if qblock_start is None or qblock_len is None:
         raise ValueError("bfloat16 prefill attention needs the query blocks of the batch")

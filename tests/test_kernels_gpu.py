@@ -298,11 +298,19 @@ def test_attention_decode_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=5, waves=3)
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=24, waves=8)
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2, 600], lens=[1, 1, 1], decode=True, pages_per_block=16, waves=4)
+    if D == 128:
+        # pages by way of LDS: blocks of up to 4 and of up to 8 waves, whole and partly filled pages, splits
+        for pages, waves in ((64, 8), (64, 3), (5, 2), (2, 1), (16, 4)):
+            attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2, 600, 63, 64, 190], lens=[1, 1, 1, 1, 1, 1], decode=True,
+                           pages_per_block=pages, waves=waves, staged=True)
 
 
 @pytest.mark.parametrize("dtype,decode", [(torch.float32, False), (torch.bfloat16, False), (torch.bfloat16, True)])
 def test_attention_far_key_and_window(ops, dtype, decode):
     lens = [1, 1] if decode else [40, 3]
+    if decode:
+        attention_case(ops, dtype, 8, 2, 128, starts=[900, 130], lens=lens, decode=True, spike=True, staged=True)
+        attention_case(ops, dtype, 8, 2, 128, starts=[900, 130], lens=lens, decode=True, window=70, staged=True)
     attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, spike=True)
     attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=100)
     attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=64, scale=0.3)
