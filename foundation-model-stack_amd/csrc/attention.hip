@@ -102,22 +102,20 @@ __device__ __forceinline__ bf16x8 load_bf16x8(const bf16* p) { return *reinterpr
 // scale2 = softmax scale * log2(e): scores and running maxima live in the base-2 domain (exp2 is the
 // hardware's native exponential).  `full`: every one of the 32 keys is visible to every column of the
 // wave, so no mask is applied (true for all but the steps at the causal edge or a window's edge).
+// The three parts of a step: scores S^T = K Q^T of 32 keys (matrix unit), the online softmax of those scores
+// (vector unit), and O^T += V^T P^T (matrix unit).
 template <int MAXDT, int QT>
-__device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
-                                          const int (&qpos)[QT], const int (&qlo)[QT], int key0, const bf16* kbase,
-                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, float scale2,
-                                          bool full) {
+__device__ __forceinline__ void step_scores(f32x4 (&sa)[QT], f32x4 (&sb)[QT], const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
+                                            const bf16* kbase, int k_stride, int head_dim) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
-  const int ndt = head_dim / 16;
   const int nchunk = (head_dim + 31) / 32;
   // Which key sits in which row of the two score tiles is free, as long as the second product pairs every
   // probability with its value.  Rows are dealt so that lane group g ends up with the probabilities of the
   // 8 consecutive keys 8 g .. 8 g + 7 (tile a: 8 g + i, tile b: 8 g + 4 + i): their values are then one
   // 16-byte read per row of the transposed values.
   const int key_a = (r >> 2) * 8 + (r & 3);
-  f32x4 sa[QT], sb[QT];
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     sa[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -139,7 +137,14 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
       }
     }
   }
-  bf16x8 pmat[QT];
+}
+
+template <int MAXDT, int QT>
+__device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&sa)[QT], f32x4 (&sb)[QT],
+                                             bf16x8 (&pmat)[QT], const int (&qpos)[QT], const int (&qlo)[QT], int key0,
+                                             int head_dim, float scale2, bool full) {
+  const int g = (threadIdx.x & (WAVE - 1)) >> 4;
+  const int ndt = head_dim / 16;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
     float mx = -INFINITY;
@@ -183,6 +188,15 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
         if (dt < ndt) st.acc[qt][dt] *= alpha;
     }
   }
+}
+
+template <int MAXDT, int QT>
+__device__ __forceinline__ void step_accumulate(WaveState<MAXDT, QT>& st, const bf16x8 (&pmat)[QT], const bf16* vbase,
+                                                int v_stride, int head_dim) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int r = lane & 15;
+  const int g = lane >> 4;
+  const int ndt = head_dim / 16;
 #pragma unroll
   for (int dt = 0; dt < MAXDT; ++dt) {
     if (dt < ndt) {
@@ -192,6 +206,18 @@ __device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8
         st.acc[qt][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v, pmat[qt], st.acc[qt][dt], 0, 0, 0);
     }
   }
+}
+
+template <int MAXDT, int QT>
+__device__ __forceinline__ void half_step(WaveState<MAXDT, QT>& st, const bf16x8 (&qreg)[QT][(MAXDT + 1) / 2],
+                                          const int (&qpos)[QT], const int (&qlo)[QT], int key0, const bf16* kbase,
+                                          int k_stride, const bf16* vbase, int v_stride, int head_dim, float scale2,
+                                          bool full) {
+  f32x4 sa[QT], sb[QT];
+  bf16x8 pmat[QT];
+  step_scores<MAXDT, QT>(sa, sb, qreg, kbase, k_stride, head_dim);
+  step_softmax<MAXDT, QT>(st, sa, sb, pmat, qpos, qlo, key0, head_dim, scale2, full);
+  step_accumulate<MAXDT, QT>(st, pmat, vbase, v_stride, head_dim);
 }
 
 // The pages page_first, page_first + page_step, ... of a sequence, straight from global memory.
@@ -429,8 +455,11 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     __syncthreads();
     if (pi < page_last) fetch(pi + 1);  // in flight while this page is multiplied
     if (has_work) {
+      // One half at a time, not unrolled: the operands of one half fill the registers.  (Both halves in one
+      // piece, with the second half's scores under way during the first half's softmax, needed more than the
+      // 256 registers that two waves per SIMD leave, and was slower with one wave as with spills.)
 #pragma unroll 1
-      for (int half = 0; half < 2; ++half) {  // not unrolled: the operands of one half fill the registers
+      for (int half = 0; half < 2; ++half) {
         const int key0 = pi * PAGE_TOKENS + half * 32;
         if (key0 > wave_hi || key0 + 31 < wave_lo) continue;  // uniform over the wave
         half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + half * 32 * KS, KS, vs + half * 32, VS, head_dim,
