@@ -147,35 +147,33 @@ __device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&s
   const int ndt = head_dim / 16;
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
+    // maxima of the raw scores, scaled once (the scale is positive); every probability is then one fused
+    // multiply-add and one exponential: exp2(s * scale2 - m)
     float mx = -INFINITY;
     if (full) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sa[qt][i] *= scale2;
-        sb[qt][i] *= scale2;
-        mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
-      }
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int ja = key0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
-        sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] * scale2 : -INFINITY;
-        sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] * scale2 : -INFINITY;
+        sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] : -INFINITY;
+        sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] : -INFINITY;
         mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
       }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(st.m[qt], mx);
+    const float m_new = fmaxf(st.m[qt], mx * scale2);
     const float alpha = __builtin_amdgcn_exp2f(st.m[qt] - m_new);
     st.m[qt] = m_new;
     float psum = 0.f;
     float pa[4], pb[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      pa[i] = __builtin_amdgcn_exp2f(sa[qt][i] - m_new);
-      pb[i] = __builtin_amdgcn_exp2f(sb[qt][i] - m_new);
+      pa[i] = __builtin_amdgcn_exp2f(fmaf(sa[qt][i], scale2, -m_new));
+      pb[i] = __builtin_amdgcn_exp2f(fmaf(sb[qt][i], scale2, -m_new));
       psum += pa[i] + pb[i];
     }
     st.l[qt] = st.l[qt] * alpha + psum;
@@ -351,40 +349,53 @@ __global__ void __launch_bounds__(WAVES* WAVE)
 }
 
 // ==========================================================================
-// prefill through LDS.  A block of 4 waves stages one page of keys and values
-// at a time in LDS; its waves are `hb` query heads of one kv group (they share
-// the page) times 4/hb runs of 16*QT consecutive query tokens.  The next page
-// is fetched into registers while the current one is multiplied.
+// prefill through LDS.  A block stages one page of keys and values at a time
+// in LDS.  It has four units: `hb` query heads of one kv group (they share the
+// page) times 4/hb runs of 16*QT consecutive query tokens; a unit is two waves
+// that take one half of every page each and meet at the end, which halves the
+// chain of dependent steps of the longest block of a causal step.  The next
+// page is fetched into registers while the current one is multiplied.
 // ==========================================================================
 #define LDS_PAD 8  // elements: rows 16 bytes apart from a multiple of the bank count
 
-template <int MAXDT, int QT>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+// EXACT: the head size is MAXDT * 16, known at compile time: the checks that let a smaller head size through
+// the same code (a quarter of the vector instructions of a step) fall away.
+template <int MAXDT, int QT, int UNITS, bool EXACT>
+__global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
     attn_prefill_lds_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
                             int n_qblocks, const int* __restrict__ block_table, int table_stride,
                             const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
-                            int kvheads, int head_dim, float scale, int window, int hb) {
+                            int kvheads, int head_dim_arg, float scale, int window, int hb) {
+  const int head_dim = EXACT ? MAXDT * 16 : head_dim_arg;
   constexpr int KS = MAXDT * 16 + LDS_PAD;    // LDS row stride of the key page [64][KS]
   constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
-  constexpr int CH = MAXDT / 2;               // 16-byte chunks a thread moves per page and operand (at most)
-  __shared__ __attribute__((aligned(16))) bf16 ks[PAGE_TOKENS * KS];
-  __shared__ __attribute__((aligned(16))) bf16 vs[MAXDT * 16 * VS];
+  constexpr int THREADS = UNITS * 2 * WAVE;
+  constexpr int CH = (MAXDT * 128 + THREADS - 1) / THREADS;  // 16-byte chunks a thread moves per page and operand (at most)
+  constexpr int K_ELEMS = PAGE_TOKENS * KS, V_ELEMS = MAXDT * 16 * VS;
+  // at the end the same memory carries one wave's state to its partner: UNITS waves x 64 lanes x (MAXDT * 4 + 2) floats
+  constexpr int MERGE_BYTES = UNITS * WAVE * (MAXDT * 4 + 2) * 4;
+  constexpr int STAGE_BYTES = (K_ELEMS + V_ELEMS) * 2 > MERGE_BYTES ? (K_ELEMS + V_ELEMS) * 2 : MERGE_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char stage[STAGE_BYTES];
+  bf16* const ks = reinterpret_cast<bf16*>(stage);
+  bf16* const vs = ks + K_ELEMS;
 
-  // Blocks of a causal step differ in length.  Workgroups are handed to compute units in linear order, a
-  // full round at a time, so the rounds alternate between long-first and short-first: a unit that got a
-  // long block in one round gets a short one in the next.
-  const unsigned linear = blockIdx.x + blockIdx.y * gridDim.x;
-  const int qb = ((linear / 256) & 1) ? (int)blockIdx.x : n_qblocks - 1 - (int)blockIdx.x;
+  // Blocks of a causal step differ in length, and the longest sets the time of the whole kernel: they go
+  // first (workgroups are handed out in linear order), and the short ones fill in behind them.
   const int group = nheads / kvheads;
   const int tiles = group / hb;
-  const int kh = blockIdx.y / tiles;
+  const int per_qb = kvheads * tiles;                 // blocks that share a query block
+  const int qb = n_qblocks - 1 - (int)(blockIdx.x / per_qb);
+  const int y = blockIdx.x % per_qb;
+  const int kh = y / tiles;
   const int wave = threadIdx.x / WAVE;
+  const int unit = wave % UNITS;  // which head and run of query tokens
+  const int khalf = wave / UNITS; // the two waves of a unit take the two halves (32 keys each) of every page
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
-  const int h = kh * group + (blockIdx.y % tiles) * hb + wave % hb;
+  const int h = kh * group + (y % tiles) * hb + unit % hb;
   const int t_begin = qblock_start[qb];
   const int t_end = t_begin + qblock_len[qb];
   const int seq = seq_of_token[t_begin];
@@ -393,7 +404,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
 
   // this wave's queries
-  const int t0 = t_begin + (wave / hb) * QT * 16;
+  const int t0 = t_begin + (unit / hb) * QT * 16;
   const bool has_work = t0 < t_end;
   bf16x8 qreg[QT][(MAXDT + 1) / 2];
   int qpos[QT], qlo[QT];
@@ -422,73 +433,93 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
   // cooperative copy: chunk id -> (row, 16-byte column) of the page in global memory and in LDS
   const int k_chunks = PAGE_TOKENS * head_dim / 8;  // per page; the value page has as many
   const int k_cols = head_dim / 8;
-  bf16x8 kbuf[CH], vbuf[CH];
-  auto fetch = [&](int pi) {
+  // Pages are fetched PF pages ahead of the one that is multiplied (a page's loads take longer to arrive than
+  // a page takes to multiply): PF sets of registers, used in turn.
+  constexpr int PF = 2;
+  bf16x8 kbuf[PF][CH], vbuf[PF][CH];
+  auto fetch = [&](int pi, bf16x8 (&kb)[CH], bf16x8 (&vb)[CH]) {
     const size_t phys = (size_t)bt[pi];
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      const int id = threadIdx.x + j * 256;
-      if (id < k_chunks) {
-        kbuf[j] = load_bf16x8(kp + (size_t)id * 8);  // the page is contiguous
-        vbuf[j] = load_bf16x8(vp + (size_t)id * 8);
-      }
+      const int id = threadIdx.x + j * THREADS;
+      const size_t at = id < k_chunks ? (size_t)id * 8 : 0;  // the page is contiguous; never a load behind a branch
+      kb[j] = load_bf16x8(kp + at);
+      vb[j] = load_bf16x8(vp + at);
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](const bf16x8 (&kb)[CH], const bf16x8 (&vb)[CH]) {
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
-      const int id = threadIdx.x + j * 256;
+      const int id = threadIdx.x + j * THREADS;
       if (id < k_chunks) {
-        *reinterpret_cast<bf16x8*>(ks + (id / k_cols) * KS + (id % k_cols) * 8) = kbuf[j];
-        *reinterpret_cast<bf16x8*>(vs + (id / 8) * VS + (id % 8) * 8) = vbuf[j];
+        *reinterpret_cast<bf16x8*>(ks + (id / k_cols) * KS + (id % k_cols) * 8) = kb[j];
+        *reinterpret_cast<bf16x8*>(vs + (id / 8) * VS + (id % 8) * 8) = vb[j];
       }
     }
   };
 
   WaveState<MAXDT, QT> st;
   wave_state_init(st);
-  fetch(page_first);
-  for (int pi = page_first; pi <= page_last; ++pi) {
-    stash();
-    __syncthreads();
-    if (pi < page_last) fetch(pi + 1);  // in flight while this page is multiplied
-    if (has_work) {
-      // One half at a time, not unrolled: the operands of one half fill the registers.  (Both halves in one
-      // piece, with the second half's scores under way during the first half's softmax, needed more than the
-      // 256 registers that two waves per SIMD leave, and was slower with one wave as with spills.)
-#pragma unroll 1
-      for (int half = 0; half < 2; ++half) {
-        const int key0 = pi * PAGE_TOKENS + half * 32;
-        if (key0 > wave_hi || key0 + 31 < wave_lo) continue;  // uniform over the wave
-        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + half * 32 * KS, KS, vs + half * 32, VS, head_dim,
+  // (a fetch past the last page reads the last page again: cheaper than a branch around loads, behind which
+  // the compiler loses count of the loads in flight and waits for all of them)
+#pragma unroll
+  for (int d = 0; d < PF; ++d) fetch(page_first + d <= page_last ? page_first + d : page_last, kbuf[d], vbuf[d]);
+  for (int p0 = page_first; p0 <= page_last; p0 += PF) {
+#pragma unroll
+    for (int d = 0; d < PF; ++d) {
+      const int pi = p0 + d;
+      if (pi > page_last) break;  // uniform
+      stash(kbuf[d], vbuf[d]);
+      block_sync_lds();  // not __syncthreads(): the pages under way must not be waited for
+      fetch(pi + PF <= page_last ? pi + PF : page_last, kbuf[d], vbuf[d]);
+      const int key0 = pi * PAGE_TOKENS + khalf * 32;
+      if (has_work && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
+        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + khalf * 32 * KS, KS, vs + khalf * 32, VS, head_dim,
                              scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
-      }
+      block_sync_lds();  // the page is overwritten next
     }
-    __syncthreads();  // the page is overwritten next
   }
 
-  if (!has_work) return;
+  // ---- the two waves of a unit meet: the second hands its state over, one run of 16 columns at a time ----
   const int ndt = head_dim / 16;
+  float* const hand = reinterpret_cast<float*>(stage) + (size_t)(unit * WAVE + lane) * (MAXDT * 4 + 2);
 #pragma unroll
   for (int qt = 0; qt < QT; ++qt) {
-    float l = st.l[qt];
-    l += __shfl_xor(l, 16, WAVE);
-    l += __shfl_xor(l, 32, WAVE);
-    const int t = t0 + qt * 16 + r;
-    if (t < t_end) {
-      const float inv = l > 0.f ? 1.f / l : 0.f;
-      bf16* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+    if (khalf == 1) {
 #pragma unroll
-      for (int dt = 0; dt < MAXDT; ++dt) {
-        if (dt < ndt) {
-          const f32x4 a = st.acc[qt][dt];
-          const bf16x4 o = {(bf16)(a[0] * inv), (bf16)(a[1] * inv), (bf16)(a[2] * inv), (bf16)(a[3] * inv)};
-          *reinterpret_cast<bf16x4*>(orow + dt * 16 + g * 4) = o;
+      for (int dt = 0; dt < MAXDT; ++dt)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) hand[dt * 4 + i] = st.acc[qt][dt][i];
+      hand[MAXDT * 4] = st.m[qt];
+      hand[MAXDT * 4 + 1] = st.l[qt];
+    }
+    __syncthreads();
+    if (khalf == 0 && has_work) {
+      const float m1 = hand[MAXDT * 4], l1 = hand[MAXDT * 4 + 1];
+      const float m = fmaxf(st.m[qt], m1);
+      const float f0 = __builtin_amdgcn_exp2f(st.m[qt] - m), f1 = __builtin_amdgcn_exp2f(m1 - m);  // base-2 maxima
+      float l = st.l[qt] * f0 + l1 * f1;
+      l += __shfl_xor(l, 16, WAVE);
+      l += __shfl_xor(l, 32, WAVE);
+      const int t = t0 + qt * 16 + r;
+      if (t < t_end) {
+        const float inv = l > 0.f ? 1.f / l : 0.f;
+        bf16* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+#pragma unroll
+        for (int dt = 0; dt < MAXDT; ++dt) {
+          if (dt < ndt) {
+            const f32x4 a = st.acc[qt][dt];
+            const float* b = hand + dt * 4;
+            const bf16x4 o = {(bf16)((a[0] * f0 + b[0] * f1) * inv), (bf16)((a[1] * f0 + b[1] * f1) * inv),
+                              (bf16)((a[2] * f0 + b[2] * f1) * inv), (bf16)((a[3] * f0 + b[3] * f1) * inv)};
+            *reinterpret_cast<bf16x4*>(orow + dt * 16 + g * 4) = o;
+          }
         }
       }
     }
+    __syncthreads();  // the memory carries the next run
   }
 }
 
@@ -524,40 +555,40 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
     float mx = -INFINITY;
     if (k0 + 31 <= qpos && k0 >= qlo) {  // uniform: all 32 keys are visible
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sa[i] *= scale2;
-        sb[i] *= scale2;
-        mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
-      }
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int ja = k0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
-        sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] * scale2 : -INFINITY;
-        sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] * scale2 : -INFINITY;
+        sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] : -INFINITY;
+        sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] : -INFINITY;
         mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
       }
     }
     mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
     mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(st.m[0], mx);
+    const float m_new = fmaxf(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
     const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
     st.m[0] = m_new;
     float pa[4], pb[4], psum = 0.f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      pa[i] = __builtin_amdgcn_exp2f(sa[i] - m_new);
-      pb[i] = __builtin_amdgcn_exp2f(sb[i] - m_new);
+      pa[i] = __builtin_amdgcn_exp2f(fmaf(sa[i], scale2, -m_new));
+      pb[i] = __builtin_amdgcn_exp2f(fmaf(sb[i], scale2, -m_new));
       psum += pa[i] + pb[i];
     }
     st.l[0] = st.l[0] * alpha + psum;
     const bf16x8 pmat = {(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3],
                          (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
+    if (__any(alpha != 1.f)) {  // the running maximum seldom moves after the first keys
+#pragma unroll
+      for (int dt = 0; dt < MAXDT; ++dt)
+        if (dt < ndt) st.acc[0][dt] *= alpha;
+    }
 #pragma unroll
     for (int dt = 0; dt < MAXDT; ++dt) {
-      if (dt < ndt)
-        st.acc[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[hf][dt], pmat, st.acc[0][dt] * alpha, 0, 0, 0);
+      if (dt < ndt) st.acc[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[hf][dt], pmat, st.acc[0][dt], 0, 0, 0);
     }
   }
 }
@@ -842,9 +873,10 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
 }
 
 // How the bfloat16 prefill kernel cuts a step: the heads of a kv group that share a block, and the
-// query tokens a block covers.  Head sizes up to 128 go through LDS (4 waves = hb heads x 4/hb runs of
+// query tokens a block covers.  Head sizes up to 128 go through LDS (4 units = hb heads x 4/hb runs of
 // 32 tokens); larger ones keep the direct kernel (128 tokens).
 #define LDS_QT 2
+#define LDS_UNITS 4  // units of a block: heads of a kv group (at most) times runs of query tokens
 static void prefill_shape(int nheads, int kvheads, int head_dim, int n_tokens, int* hb, int* qt, int* qblock) {
   const int group = nheads / kvheads;
   (void)n_tokens;
@@ -852,9 +884,9 @@ static void prefill_shape(int nheads, int kvheads, int head_dim, int n_tokens, i
     *hb = 1, *qt = 0, *qblock = PREFILL_QBLOCK;
     return;
   }
-  *hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
+  *hb = (LDS_UNITS >= 4 && group % 4 == 0) ? 4 : (group % 2 == 0 ? 2 : 1);
   *qt = LDS_QT;
-  *qblock = (4 / *hb) * *qt * 16;
+  *qblock = (LDS_UNITS / *hb) * *qt * 16;
 }
 
 extern "C" int fmsamd_attn_prefill_qblock(int nheads, int kvheads, int head_dim, int n_tokens) {
@@ -886,15 +918,26 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
     FMS_LAUNCH_CHECK("attn_prefill_bf16");
     return 0;
   }
-  const int hb = group % 4 == 0 ? 4 : (group % 2 == 0 ? 2 : 1);
-  FMS_REQUIRE(qblock_tokens == (4 / hb) * LDS_QT * 16, "attn_prefill_bf16: query blocks of %d tokens, %d expected",
-              qblock_tokens, (4 / hb) * LDS_QT * 16);
-  dim3 grid(n_qblocks, kvheads * (group / hb));
+  int hb, qt_unused, qblock_expected;
+  prefill_shape(nheads, kvheads, head_dim, n_tokens, &hb, &qt_unused, &qblock_expected);
+  FMS_REQUIRE(qblock_tokens == qblock_expected, "attn_prefill_bf16: query blocks of %d tokens, %d expected",
+              qblock_tokens, qblock_expected);
+  const long blocks = (long)n_qblocks * kvheads * (group / hb);
+  FMS_REQUIRE(blocks < (1l << 31), "attn_prefill_bf16: %ld blocks exceed one launch", blocks);
+  dim3 grid((unsigned)blocks);
 #define FMS_PL(M)                                                                                                  \
-  attn_prefill_lds_kernel<M, LDS_QT><<<grid, dim3(256), 0, stream>>>(                                              \
+  do {                                                                                                             \
+  if (head_dim == M * 16)                                                                                          \
+    attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, true><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(          \
+        (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,       \
+        n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads,         \
+        head_dim, scale, window, hb);                                                                              \
+  else                                                                                                             \
+    attn_prefill_lds_kernel<M, LDS_QT, LDS_UNITS, false><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(         \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len,         \
       n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
-      scale, window, hb)
+      scale, window, hb);                                                                                          \
+  } while (0)
   if (head_dim <= 64)
     FMS_PL(4);
   else

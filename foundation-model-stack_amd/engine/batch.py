@@ -20,7 +20,8 @@ class StepBatch:
     q_lens: List[int]  # tokens each sequence brings
     starts: List[int]  # position of each sequence's first token
     is_decode: bool  # every sequence brings exactly one token
-    max_context: int  # longest sequence after this step (host value, bounds the decode split)
+    max_context: int  # longest sequence after this step (host value)
+    context_bound: int  # what the decode attention is launched for: max_context or a rounder number above it
     token_ids: torch.Tensor  # int32 [T]
     positions: torch.Tensor  # int32 [T]
     seq_of_token: torch.Tensor  # int32 [T], index into the rows of the block tables (-1: padding row)
@@ -105,6 +106,7 @@ def build_batch(
         starts=list(starts),
         is_decode=all(n == 1 for n in q_lens),
         max_context=max(s + n for s, n in zip(starts, q_lens)),
+        context_bound=max(s + n for s, n in zip(starts, q_lens)),
         token_ids=span(0),
         positions=span(1),
         seq_of_token=span(2),

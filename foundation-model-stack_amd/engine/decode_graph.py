@@ -63,7 +63,7 @@ class DecodeGraph:
         self.rng = torch.zeros(rows, 2, dtype=torch.int64, device=dev)
         self.batch = StepBatch(
             n_tokens=rows, n_seqs=rows, slots=[], q_lens=[1] * rows, starts=[0] * rows, is_decode=True,
-            max_context=max_context, token_ids=self.tokens, positions=self.positions, seq_of_token=self.seq_of_token,
+            max_context=max_context, context_bound=max_context, token_ids=self.tokens, positions=self.positions, seq_of_token=self.seq_of_token,
             slot_ids=self.slot_ids, seq_starts=self.seq_starts, block_tables=self.tables,
             logit_rows=self.logit_rows, n_logit_rows=rows,
         )

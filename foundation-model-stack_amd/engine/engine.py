@@ -156,4 +156,9 @@ class Engine:
                 size = block.mixer.prefill_qblock(n_tokens, self.model.dtype)
                 if size:
                     sizes.add(size)
-        return build_batch(self.cache, slots, tokens, starts, want, self.device, sizes)
+        batch = build_batch(self.cache, slots, tokens, starts, want, self.device, sizes)
+        if batch.is_decode:
+            # the bound a graph for this step would be captured for: eager steps and replays then launch the
+            # same kernels in the same shape, and give the same bits
+            batch.context_bound = context_bucket(batch.max_context + CONTEXT_HEADROOM, self.cache.max_seq_len)
+        return batch

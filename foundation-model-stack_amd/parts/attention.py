@@ -105,7 +105,7 @@ class MultiHeadAttention(Mixer):
         qb_start, qb_len = batch.qblocks.get(size, (None, None))
         mixed = ops.attention(
             qkv, batch.positions, batch.seq_of_token, table, cache.keys, cache.values, H, K, D, self.scale, self.window,
-            decode=batch.is_decode, max_context=batch.max_context,
+            decode=batch.is_decode, max_context=batch.context_bound,
             qblock_start=qb_start, qblock_len=qb_len, qblock_tokens=size,
         )
         return BranchOutput(mixed, self.dense)
