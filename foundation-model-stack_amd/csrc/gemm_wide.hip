@@ -72,22 +72,26 @@ __global__ void __launch_bounds__(512)
 
   // WD_DEPTH steps in flight: while step t multiplies, the loads of steps t + 1 .. t + WD_DEPTH - 1 are under
   // way (a load takes several steps' time to arrive)
+  // Every step issues the loads of the step WD_DEPTH - 1 ahead, in range or not (past the slice's end the last
+  // step is loaded again and never used): with the same number of loads under way wherever the loop is, the
+  // compiler can wait for exactly the oldest ones instead of for all.
   bf16x8 xr[WD_DEPTH][XP], wr[WD_DEPTH][4];
+  const int g_last = g_end - 1;
 #pragma unroll
-  for (int d = 0; d < WD_DEPTH - 1; ++d)
-    if (g_begin + d < g_end) {
-      load_x(g_begin + d, xr[d]);
-      load_w(g_begin + d, wr[d]);
-    }
+  for (int d = 0; d < WD_DEPTH - 1; ++d) {
+    const int at = g_begin + d < g_end ? g_begin + d : g_last;
+    load_x(at, xr[d]);
+    load_w(at, wr[d]);
+  }
   for (int grp = g_begin; grp < g_end; grp += WD_DEPTH) {
 #pragma unroll
     for (int d = 0; d < WD_DEPTH; ++d) {
       const int cur = grp + d;
-      if (cur >= g_end) break;  // uniform
       constexpr int ahead = WD_DEPTH - 1;
-      if (cur + ahead < g_end) {
-        load_x(cur + ahead, xr[(d + ahead) % WD_DEPTH]);
-        load_w(cur + ahead, wr[(d + ahead) % WD_DEPTH]);
+      {
+        const int at = cur + ahead < g_end ? cur + ahead : g_last;
+        load_x(at, xr[(d + ahead) % WD_DEPTH]);
+        load_w(at, wr[(d + ahead) % WD_DEPTH]);
       }
       const int buf = d & 1;  // WD_DEPTH is even: steps alternate between the two x buffers
       store_x(cur, buf, xr[d]);
@@ -97,24 +101,26 @@ __global__ void __launch_bounds__(512)
         *reinterpret_cast<bf16x8*>(ws[wave] + row * WD_GROUP + ((seg ^ row) & 15) * 8) = w_ok(cur, q) ? wr[d][q] : zero;
       }
       block_sync_lds();  // the step's x is whole; the buffer written now was last read two steps ago
-      bf16x8 a[4];
+      if (cur < g_end) {  // uniform; a step past the end multiplies nothing
+        bf16x8 a[4];
 #pragma unroll
-      for (int st = 0; st < 4; ++st)
-        a[st] = *reinterpret_cast<const bf16x8*>(ws[wave] + r * WD_GROUP + (((st * 4 + g) ^ r) & 15) * 8);
-      // all operands of the step first, then the products: a read that waits in front of every product
-      // would pay the LDS latency sixteen times a step
-      bf16x8 b[MT][4];
+        for (int st = 0; st < 4; ++st)
+          a[st] = *reinterpret_cast<const bf16x8*>(ws[wave] + r * WD_GROUP + (((st * 4 + g) ^ r) & 15) * 8);
+        // all operands of the step first, then the products: a read that waits in front of every product
+        // would pay the LDS latency sixteen times a step
+        bf16x8 b[MT][4];
 #pragma unroll
-      for (int j = 0; j < MT; ++j)
+        for (int j = 0; j < MT; ++j)
 #pragma unroll
-        for (int st = 0; st < 4; ++st) {
-          const int m = j * 16 + r;
-          b[j][st] = *reinterpret_cast<const bf16x8*>(xs[buf] + m * WD_GROUP + (((st * 4 + g) ^ m) & 15) * 8);
-        }
+          for (int st = 0; st < 4; ++st) {
+            const int m = j * 16 + r;
+            b[j][st] = *reinterpret_cast<const bf16x8*>(xs[buf] + m * WD_GROUP + (((st * 4 + g) ^ m) & 15) * 8);
+          }
 #pragma unroll
-      for (int j = 0; j < MT; ++j)
+        for (int j = 0; j < MT; ++j)
 #pragma unroll
-        for (int st = 0; st < 4; ++st) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[st], b[j][st], acc[j], 0, 0, 0);
+          for (int st = 0; st < 4; ++st) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[st], b[j][st], acc[j], 0, 0, 0);
+      }
     }
   }
   // acc[j][e]: weight row n0 + 4 g + e, x row 16 j + r
@@ -214,17 +220,27 @@ __global__ void __launch_bounds__(256)
   }
 }
 
-// Slices of K: enough blocks for all compute units, and no slice under two steps.
-static int wide_slices(int rows, int K) {
+// Slices of K.  A block's time goes with its steps; the blocks run in rounds over the compute units; and the
+// partial sums are written and read once per slice.  The number of slices with the least of
+//   rounds x steps per slice + (partial bytes a compute unit moves) / (bytes of a step)
+// wins: 48 blocks of rows in 5 slices are one round of 7 steps, in 6 slices two rounds of 6.
+static int wide_slices(int M, int rows, int K) {
   const int row_blocks = ceil_div(rows, WD_ROWS);
   const int ngroups = ceil_div(K, WD_GROUP);
-  int slices = ceil_div(WD_COMPUTE_UNITS, row_blocks);
-  if (slices > ngroups / 2) slices = ngroups / 2;
-  return slices < 1 ? 1 : slices;
+  int best = 1;
+  double best_cost = 0;
+  for (int slices = 1; slices <= ngroups && slices <= 64; ++slices) {
+    const double rounds = ceil_div((long)row_blocks * slices, WD_COMPUTE_UNITS);
+    const double steps = ceil_div(ngroups, slices);
+    const double partial = (double)slices * M * rows * 8 / WD_COMPUTE_UNITS / (WD_ROWS * WD_GROUP * 2);
+    const double cost = rounds * steps + partial + 1.0;  // + a step's worth of start and end per slice's block
+    if (slices == 1 || cost < best_cost) best = slices, best_cost = cost;
+  }
+  return best;
 }
 
 long wide_workspace_bytes(int M, int rows, int K) {
-  return (long)wide_slices(rows, K) * M * rows * (long)sizeof(float);
+  return (long)wide_slices(M, rows, K) * M * rows * (long)sizeof(float);
 }
 
 template <int EPI>
@@ -258,7 +274,7 @@ int wide_product(int epi, const void* x, long ldx, const void* w, const void* bi
   FMS_REQUIRE(M > 16 && M <= 64, "wide product: %d rows (17..64)", M);
   FMS_REQUIRE(workspace != nullptr && workspace_bytes >= wide_workspace_bytes(M, rows, K),
               "wide product: workspace of %ld bytes, %ld needed", workspace_bytes, wide_workspace_bytes(M, rows, K));
-  const int slices = wide_slices(rows, K);
+  const int slices = wide_slices(M, rows, K);
   const int ngroups = ceil_div(K, WD_GROUP);
   const int per_slice = ceil_div(ngroups, slices);
   dim3 grid(ceil_div(rows, WD_ROWS), slices);
