@@ -723,12 +723,12 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   const int kh = blockIdx.y / tiles_per_kv;
   const int ht = blockIdx.y % tiles_per_kv;
   const int t = blockIdx.z;
-  const int wave = threadIdx.x / WAVE;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);  // uniform: table entries load as scalars
   const int n_waves = blockDim.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
-  const int seq = seq_of_token[t];
+  const int seq = uniform_load(seq_of_token + t);
   const int cols = group - ht * tile_cols < tile_cols ? group - ht * tile_cols : tile_cols;  // query heads here
   const int head0 = kh * group + ht * tile_cols;
   if (seq < 0) {
@@ -737,7 +737,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
         out[(size_t)t * out_stride + (size_t)head0 * head_dim + i] = (bf16)0.f;
     return;
   }
-  const int pos = positions[t];
+  const int pos = uniform_load(positions + t);
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   int page_lo, page_hi;
   if (split >= split_pages(lo, pos, n_splits, split, &page_lo, &page_hi)) return;
@@ -751,7 +751,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   WaveState<MAXDT, 1> st;
   wave_state_init(st);
   for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
-    const size_t phys = (size_t)bt[pi];
+    const size_t phys = (size_t)uniform_load(bt + pi);
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
     if (STAGED) {

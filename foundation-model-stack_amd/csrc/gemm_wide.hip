@@ -3,33 +3,95 @@
 // With this many rows of x the activations are no longer small beside the weights: a block that owns 16
 // weight rows and all of K (gemm.hip) reads four times as many bytes of x as of W.  Here a block owns 128
 // weight rows (a 16-row tile per wave) and a slice of K, and its waves share the x rows of the slice through
-// LDS, so x is read once per 128 weight rows.  The price is that the slices of K meet in memory: the
-// product kernel leaves float32 partial sums in a workspace, and a second kernel adds them in a fixed order
-// (the same bits whatever the launch looks like) and applies the epilogue.
+// LDS, so x is read once per 128 weight rows.  When K has to be cut into slices to fill the compute units,
+// the slices meet in memory: the product kernel leaves float32 partial sums in a workspace, and a second
+// kernel adds them in a fixed order (the same bits whatever the launch looks like) and applies the epilogue.
+// A product with enough weight rows for one slice (the gated feed-forward product, the output head) is
+// finished by the product kernel itself.
 #include "gemm_epilogue.h"
 
 #define WD_ROWS 128   // weight rows per block
 #define WD_GROUP 128  // k-values per step of the stream
 #define WD_COMPUTE_UNITS 256
-#define WD_DEPTH 4  // steps whose loads are in flight (even)
+#define WD_DEPTH 4       // steps whose loads are in flight (even)
+#define WD_TILE_LD 132   // floats per row of the block's result tile in LDS: 128 and a shift of the banks
+
+// What the product kernel does with its block's result tile.
+#define WD_PARTIAL 0  // a slice of K: float32 partial sums into the workspace
+#define WD_PLAIN 1    // all of K: row scale, bias, store
+#define WD_GATED 2    // all of K; the block owns 64 gate rows and their 64 up rows: act(gate) * up
+
+struct WideOut {
+  void* out;
+  long ldo;
+  const void* bias;
+  int bias_f32;
+  int N, tile2_offset, act;
+  int vec;  // rows of the destination start 16-byte aligned: four elements at a time
+  RowScale scale;
+};
+
+__device__ __forceinline__ float wide_bias(const WideOut& o, int n) {
+  return o.bias_f32 ? ((const float*)o.bias)[n] : to_f32(((const bf16*)o.bias)[n]);
+}
+__device__ __forceinline__ void store4(float* p, f32x4 v) { *reinterpret_cast<f32x4*>(p) = v; }
+__device__ __forceinline__ void store4(bf16* p, f32x4 v) {
+  const bf16x4 b = {(bf16)v[0], (bf16)v[1], (bf16)v[2], (bf16)v[3]};
+  *reinterpret_cast<bf16x4*>(p) = b;
+}
 
 // Loads are 16 rows' 256 contiguous bytes as 4 instructions of 4 rows (what the memory system streams at
 // full rate); LDS holds them as loaded, with the 16-byte pieces of a row XOR-swizzled by the row, and gives
 // them back in the MFMA operand layout (lane (r, g) takes row r, k-step s at piece 4 s + g).
-template <int MT>
+template <int MT, int MODE, typename OutT>
 __global__ void __launch_bounds__(512)
-    wide_partial_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, float* __restrict__ part,
-                        int M, int rows, int K, int groups_per_slice) {
-  __shared__ __attribute__((aligned(16))) bf16 xs[2][MT * 16 * WD_GROUP];  // two steps of x: one read, one written
-  __shared__ __attribute__((aligned(16))) bf16 ws[8][16 * WD_GROUP];       // a wave's own weight tile
+    wide_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, float* __restrict__ part, int M,
+                int rows, int K, int groups_per_slice, WideOut o) {
+  constexpr int XS_BYTES = 2 * MT * 16 * WD_GROUP * 2;  // two steps of x: one read, one written
+  constexpr int WS_BYTES = 8 * 16 * WD_GROUP * 2;       // a weight tile per wave
+  constexpr int TILE_BYTES = MT * 16 * WD_TILE_LD * 4;  // the block's results, once the stream has ended
+  constexpr int SMEM = XS_BYTES + WS_BYTES > TILE_BYTES ? XS_BYTES + WS_BYTES : TILE_BYTES;
+  __shared__ __attribute__((aligned(16))) char smem[SMEM];
+  __shared__ float row_scale[MT * 16];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
+  bf16* const xs = reinterpret_cast<bf16*>(smem);
+  bf16* const ws = reinterpret_cast<bf16*>(smem + XS_BYTES) + wave * 16 * WD_GROUP;
+  float* const tile = reinterpret_cast<float*>(smem);
   const int r = lane & 15, g = lane >> 4;
   const int lrow = lane >> 4, seg = lane & 15;
-  const int n0 = blockIdx.x * WD_ROWS + wave * 16;
+  // the wave's 16 weight rows start at n0; rows from n_end on are not the wave's to read
+  int n0 = blockIdx.x * WD_ROWS + wave * 16, n_end = rows;
+  if (MODE == WD_GATED) {
+    const int first = blockIdx.x * (WD_ROWS / 2) + (wave & 3) * 16;
+    n0 = wave < 4 ? first : o.tile2_offset + first;
+    n_end = wave < 4 ? o.N : o.tile2_offset + o.N;
+  }
   const int ngroups = (K + WD_GROUP - 1) / WD_GROUP;
   const int g_begin = blockIdx.y * groups_per_slice;
   const int g_end = g_begin + groups_per_slice < ngroups ? g_begin + groups_per_slice : ngroups;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  if (MODE != WD_PARTIAL) {  // 1 / rms of the rows of x, if their norm was left to this product
+    constexpr int RPW = MT * 2;
+    if (o.scale.partials != nullptr) {
+      float sum[RPW];
+#pragma unroll
+      for (int k = 0; k < RPW; ++k) sum[k] = 0.f;
+      for (int i = lane; i < o.scale.count; i += WAVE)
+#pragma unroll
+        for (int k = 0; k < RPW; ++k) {
+          const int m = wave * RPW + k < M ? wave * RPW + k : M - 1;
+          sum[k] += o.scale.partials[(size_t)m * o.scale.count + i];
+        }
+#pragma unroll
+      for (int k = 0; k < RPW; ++k) {
+        const float total = wave_sum(sum[k]);
+        if (lane == 0) row_scale[wave * RPW + k] = rsqrtf(total * o.scale.inv_width + o.scale.eps);
+      }
+    } else if (lane < RPW) {
+      row_scale[wave * RPW + lane] = 1.f;
+    }
+  }
 
   // x pieces of a step: MT * 16 rows x 16 pieces, dealt over the 512 threads (row = id / 16, piece = id % 16).
   // Loads never sit behind a branch and their data is not touched before the step that uses it (either makes
@@ -40,7 +102,7 @@ __global__ void __launch_bounds__(512)
     const int id = threadIdx.x + i * 512;
     return id < MT * 256 && (id >> 4) < M && grp * WD_GROUP + (id & 15) * 8 < K;
   };
-  auto w_ok = [&](int grp, int q) { return n0 + 4 * q + lrow < rows && grp * WD_GROUP + seg * 8 < K; };
+  auto w_ok = [&](int grp, int q) { return n0 + 4 * q + lrow < n_end && grp * WD_GROUP + seg * 8 < K; };
   auto load_x = [&](int grp, bf16x8 (&xr)[XP]) {
 #pragma unroll
     for (int i = 0; i < XP; ++i) {
@@ -55,7 +117,8 @@ __global__ void __launch_bounds__(512)
       const int id = threadIdx.x + i * 512;
       const int m = id >> 4, piece = id & 15;
       if (id < MT * 256)
-        *reinterpret_cast<bf16x8*>(xs[buf] + m * WD_GROUP + ((piece ^ m) & 15) * 8) = x_ok(grp, i) ? xr[i] : zero;
+        *reinterpret_cast<bf16x8*>(xs + buf * (MT * 16 * WD_GROUP) + m * WD_GROUP + ((piece ^ m) & 15) * 8) =
+            x_ok(grp, i) ? xr[i] : zero;
     }
   };
   auto load_w = [&](int grp, bf16x8 (&wr)[4]) {
@@ -71,41 +134,46 @@ __global__ void __launch_bounds__(512)
   for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // WD_DEPTH steps in flight: while step t multiplies, the loads of steps t + 1 .. t + WD_DEPTH - 1 are under
-  // way (a load takes several steps' time to arrive)
-  // Every step issues the loads of the step WD_DEPTH - 1 ahead, in range or not (past the slice's end the last
-  // step is loaded again and never used): with the same number of loads under way wherever the loop is, the
-  // compiler can wait for exactly the oldest ones instead of for all.
+  // way (a load takes several steps' time to arrive).  Every step issues the loads of the step WD_DEPTH - 1
+  // ahead, in range or not (past the slice's end the last step is loaded again and never used): with the same
+  // number of loads under way wherever the loop is, the compiler can wait for exactly the oldest ones instead
+  // of for all.
+  // The blocks walk their slice from different starting steps and wrap around: blocks that all read the same
+  // 256 bytes of their rows at the same time (rows lie a multiple of kilobytes apart) crowd into few memory
+  // channels.  The start depends on the block's place only, so the order of the sum does too.
   bf16x8 xr[WD_DEPTH][XP], wr[WD_DEPTH][4];
-  const int g_last = g_end - 1;
+  const int n_steps = g_end - g_begin;
+  const int rot = (blockIdx.x * 5) % n_steps;
+  auto group_of = [&](int t) {  // the k-group of the slice's step t (steps past the end repeat the last one)
+    const int u = (t < n_steps ? t : n_steps - 1) + rot;
+    return g_begin + (u >= n_steps ? u - n_steps : u);
+  };
 #pragma unroll
   for (int d = 0; d < WD_DEPTH - 1; ++d) {
-    const int at = g_begin + d < g_end ? g_begin + d : g_last;
-    load_x(at, xr[d]);
-    load_w(at, wr[d]);
+    load_x(group_of(d), xr[d]);
+    load_w(group_of(d), wr[d]);
   }
-  for (int grp = g_begin; grp < g_end; grp += WD_DEPTH) {
+  for (int t = 0; t < n_steps; t += WD_DEPTH) {
 #pragma unroll
     for (int d = 0; d < WD_DEPTH; ++d) {
-      const int cur = grp + d;
+      const int cur = t + d;
       constexpr int ahead = WD_DEPTH - 1;
-      {
-        const int at = cur + ahead < g_end ? cur + ahead : g_last;
-        load_x(at, xr[(d + ahead) % WD_DEPTH]);
-        load_w(at, wr[(d + ahead) % WD_DEPTH]);
-      }
+      load_x(group_of(cur + ahead), xr[(d + ahead) % WD_DEPTH]);
+      load_w(group_of(cur + ahead), wr[(d + ahead) % WD_DEPTH]);
       const int buf = d & 1;  // WD_DEPTH is even: steps alternate between the two x buffers
-      store_x(cur, buf, xr[d]);
+      const int cur_g = group_of(cur);
+      store_x(cur_g, buf, xr[d]);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = 4 * q + lrow;
-        *reinterpret_cast<bf16x8*>(ws[wave] + row * WD_GROUP + ((seg ^ row) & 15) * 8) = w_ok(cur, q) ? wr[d][q] : zero;
+        *reinterpret_cast<bf16x8*>(ws + row * WD_GROUP + ((seg ^ row) & 15) * 8) = w_ok(cur_g, q) ? wr[d][q] : zero;
       }
       block_sync_lds();  // the step's x is whole; the buffer written now was last read two steps ago
-      if (cur < g_end) {  // uniform; a step past the end multiplies nothing
+      if (cur < n_steps) {  // uniform; a step past the end multiplies nothing
         bf16x8 a[4];
 #pragma unroll
         for (int st = 0; st < 4; ++st)
-          a[st] = *reinterpret_cast<const bf16x8*>(ws[wave] + r * WD_GROUP + (((st * 4 + g) ^ r) & 15) * 8);
+          a[st] = *reinterpret_cast<const bf16x8*>(ws + r * WD_GROUP + (((st * 4 + g) ^ r) & 15) * 8);
         // all operands of the step first, then the products: a read that waits in front of every product
         // would pay the LDS latency sixteen times a step
         bf16x8 b[MT][4];
@@ -114,7 +182,8 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
           for (int st = 0; st < 4; ++st) {
             const int m = j * 16 + r;
-            b[j][st] = *reinterpret_cast<const bf16x8*>(xs[buf] + m * WD_GROUP + (((st * 4 + g) ^ m) & 15) * 8);
+            b[j][st] = *reinterpret_cast<const bf16x8*>(xs + buf * (MT * 16 * WD_GROUP) + m * WD_GROUP +
+                                                        (((st * 4 + g) ^ m) & 15) * 8);
           }
 #pragma unroll
         for (int j = 0; j < MT; ++j)
@@ -123,16 +192,80 @@ __global__ void __launch_bounds__(512)
       }
     }
   }
-  // acc[j][e]: weight row n0 + 4 g + e, x row 16 j + r
-  float* dst = part + (size_t)blockIdx.y * M * rows;
+
+  // The block's results meet in LDS (where the stream's buffers were): row m of x, then the block's 128
+  // weight rows in the order of the waves; from there they leave in whole rows of 256 or 512 bytes.
+  // acc[j][e]: the wave's weight row 4 g + e, x row 16 j + r.
+  __syncthreads();
 #pragma unroll
-  for (int j = 0; j < MT; ++j) {
-    const int m = j * 16 + r;
-    if (m >= M) continue;
+  for (int j = 0; j < MT; ++j) *reinterpret_cast<f32x4*>(tile + (j * 16 + r) * WD_TILE_LD + wave * 16 + 4 * g) = acc[j];
+  __syncthreads();
+
+  if (MODE == WD_GATED) {
+    // 16 threads a row: four gate columns and their four up columns each
+    const int c = 4 * (threadIdx.x & 15);
+    const int n = blockIdx.x * (WD_ROWS / 2) + c;
+    OutT* const out = (OutT*)o.out;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int n = n0 + 4 * g + e;
-      if (n < rows) dst[(size_t)m * rows + n] = acc[j][e];
+    for (int p = 0; p < (MT + 1) / 2; ++p) {
+      const int m = p * 32 + (threadIdx.x >> 4);
+      if (m >= M || m >= MT * 16 || n >= o.N) continue;
+      const f32x4 gate = *reinterpret_cast<const f32x4*>(tile + m * WD_TILE_LD + c);
+      const f32x4 up = *reinterpret_cast<const f32x4*>(tile + m * WD_TILE_LD + WD_ROWS / 2 + c);
+      const float rs = row_scale[m];
+      f32x4 res;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        float v = gate[e] * rs, u = up[e] * rs;
+        if (o.bias != nullptr && n + e < o.N) {
+          v += wide_bias(o, n + e);
+          u += wide_bias(o, o.tile2_offset + n + e);
+        }
+        res[e] = sk_activate(v, o.act) * u;
+      }
+      if (o.vec && n + 3 < o.N) {
+        store4(out + (size_t)m * o.ldo + n, res);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < o.N) out[(size_t)m * o.ldo + n + e] = from_f32<OutT>(res[e]);
+      }
+    }
+  } else {
+    // 32 threads a row: four columns each
+    const int c = 4 * (threadIdx.x & 31);
+    const int n = blockIdx.x * WD_ROWS + c;
+    const int n_lim = MODE == WD_PLAIN ? o.N : rows;
+#pragma unroll
+    for (int p = 0; p < MT; ++p) {
+      const int m = p * 16 + (threadIdx.x >> 5);
+      if (m >= M || n >= n_lim) continue;
+      f32x4 v = *reinterpret_cast<const f32x4*>(tile + m * WD_TILE_LD + c);
+      if (MODE == WD_PLAIN) {
+        const float rs = row_scale[m];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] *= rs;
+          if (o.bias != nullptr && n + e < n_lim) v[e] += wide_bias(o, n + e);
+        }
+        OutT* const out = (OutT*)o.out;
+        if (o.vec && n + 3 < n_lim) {
+          store4(out + (size_t)m * o.ldo + n, v);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < n_lim) out[(size_t)m * o.ldo + n + e] = from_f32<OutT>(v[e]);
+        }
+      } else {
+        float* const dst = part + ((size_t)blockIdx.y * M + m) * rows + n;
+        if (o.vec && n + 3 < n_lim) {
+          store4(dst, v);
+        } else {
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (n + e < n_lim) dst[e] = v[e];
+        }
+      }
     }
   }
 }
@@ -149,17 +282,29 @@ __global__ void __launch_bounds__(256)
   if (m >= M) return;  // whole waves
   const bool live = n < N;
 
+  // The slices are added in their order, four loads under way at a time.
+  auto add_slices = [&](const float* p) {
+    const size_t stride = (size_t)M * rows;
+    float sum = 0.f;
+    int s = 0;
+    for (; s + 4 <= slices; s += 4) {
+      const float a0 = p[(size_t)s * stride], a1 = p[(size_t)(s + 1) * stride], a2 = p[(size_t)(s + 2) * stride],
+                  a3 = p[(size_t)(s + 3) * stride];
+      sum = (((sum + a0) + a1) + a2) + a3;
+    }
+    for (; s < slices; ++s) sum += p[(size_t)s * stride];
+    return sum;
+  };
+  float v = 0.f, u = 0.f;
+  if (live) {
+    v = add_slices(part + (size_t)m * rows + n);
+    if (EPI == EPI_GATED) u = add_slices(part + (size_t)m * rows + tile2_offset + n);
+  }
   float row_scale = 1.f;
   if (scale.partials != nullptr) {
     float sum = 0.f;
     for (int i = lane; i < scale.count; i += WAVE) sum += scale.partials[(size_t)m * scale.count + i];
     row_scale = rsqrtf(wave_sum(sum) * scale.inv_width + scale.eps);
-  }
-  float v = 0.f, u = 0.f;
-  if (live) {
-    for (int s = 0; s < slices; ++s) v += part[((size_t)s * M + m) * rows + n];
-    if (EPI == EPI_GATED)
-      for (int s = 0; s < slices; ++s) u += part[((size_t)s * M + m) * rows + tile2_offset + n];
   }
   v *= row_scale;
   u *= row_scale;
@@ -221,10 +366,13 @@ __global__ void __launch_bounds__(256)
 }
 
 // Slices of K.  A block's time goes with its steps; the blocks run in rounds over the compute units; and the
-// partial sums are written and read once per slice.  The number of slices with the least of
+// partial sums are written and read once per slice (not at all when the product kernel finishes its one
+// slice itself).  The number of slices with the least of
 //   rounds x steps per slice + (partial bytes a compute unit moves) / (bytes of a step)
 // wins: 48 blocks of rows in 5 slices are one round of 7 steps, in 6 slices two rounds of 6.
-static int wide_slices(int M, int rows, int K) {
+static bool wide_finishes_itself(int epi) { return epi == EPI_PLAIN || epi == EPI_GATED; }
+
+static int wide_slices(int epi, int M, int rows, int K) {
   const int row_blocks = ceil_div(rows, WD_ROWS);
   const int ngroups = ceil_div(K, WD_GROUP);
   int best = 1;
@@ -232,15 +380,17 @@ static int wide_slices(int M, int rows, int K) {
   for (int slices = 1; slices <= ngroups && slices <= 64; ++slices) {
     const double rounds = ceil_div((long)row_blocks * slices, WD_COMPUTE_UNITS);
     const double steps = ceil_div(ngroups, slices);
-    const double partial = (double)slices * M * rows * 8 / WD_COMPUTE_UNITS / (WD_ROWS * WD_GROUP * 2);
+    double partial = (double)slices * M * rows * 8 / WD_COMPUTE_UNITS / (WD_ROWS * WD_GROUP * 2);
+    if (slices == 1 && wide_finishes_itself(epi)) partial = 0;
     const double cost = rounds * steps + partial + 1.0;  // + a step's worth of start and end per slice's block
     if (slices == 1 || cost < best_cost) best = slices, best_cost = cost;
   }
   return best;
 }
 
+// Enough for any epilogue of this shape.
 long wide_workspace_bytes(int M, int rows, int K) {
-  return (long)wide_slices(M, rows, K) * M * rows * (long)sizeof(float);
+  return (long)wide_slices(EPI_RESID, M, rows, K) * M * rows * (long)sizeof(float);
 }
 
 template <int EPI>
@@ -266,27 +416,63 @@ static void launch_finish(const float* part, int slices, int rows, const void* b
 #undef FMS_WF
 }
 
+template <int MODE, typename OutT>
+static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float* part, int M, int rows, int K,
+                        int per_slice, const WideOut& o, hipStream_t stream) {
+  const int mt = ceil_div(M, 16);
+#define FMS_WK(MT) \
+  wide_kernel<MT, MODE, OutT><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice, o)
+  if (mt == 2)
+    FMS_WK(2);
+  else if (mt == 3)
+    FMS_WK(3);
+  else
+    FMS_WK(4);
+#undef FMS_WK
+}
+
+static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
 // N: columns of the output (for the gated product the hidden size; W then has tile2_offset + N rows).
 int wide_product(int epi, const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                  int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, RowScale scale,
                  RopeEpilogue rope, ResidEpilogue res, void* workspace, long workspace_bytes, hipStream_t stream) {
   const int rows = epi == EPI_GATED ? tile2_offset + N : N;
   FMS_REQUIRE(M > 16 && M <= 64, "wide product: %d rows (17..64)", M);
-  FMS_REQUIRE(workspace != nullptr && workspace_bytes >= wide_workspace_bytes(M, rows, K),
-              "wide product: workspace of %ld bytes, %ld needed", workspace_bytes, wide_workspace_bytes(M, rows, K));
-  const int slices = wide_slices(M, rows, K);
+  const int slices = wide_slices(epi, M, rows, K);
   const int ngroups = ceil_div(K, WD_GROUP);
   const int per_slice = ceil_div(ngroups, slices);
+  const bool itself = slices == 1 && wide_finishes_itself(epi);
+  WideOut o{out, ldo, bias, bias != nullptr && bias_dtype == FMS_F32, N, tile2_offset, act, 0, scale};
+
+  if (itself) {
+    const long elem = out_dtype == FMS_BF16 ? 2 : 4;
+    o.vec = ((uintptr_t)out % (4 * elem)) == 0 && ldo % 4 == 0;
+    if (epi == EPI_GATED) {
+      dim3 grid(ceil_div(N, WD_ROWS / 2), 1);
+      if (out_dtype == FMS_BF16)
+        launch_wide<WD_GATED, bf16>(grid, x, ldx, w, nullptr, M, rows, K, per_slice, o, stream);
+      else
+        launch_wide<WD_GATED, float>(grid, x, ldx, w, nullptr, M, rows, K, per_slice, o, stream);
+    } else {
+      dim3 grid(ceil_div(N, WD_ROWS), 1);
+      if (out_dtype == FMS_BF16)
+        launch_wide<WD_PLAIN, bf16>(grid, x, ldx, w, nullptr, M, rows, K, per_slice, o, stream);
+      else
+        launch_wide<WD_PLAIN, float>(grid, x, ldx, w, nullptr, M, rows, K, per_slice, o, stream);
+    }
+    FMS_LAUNCH_CHECK("wide product");
+    return 0;
+  }
+
+  const long needed = (long)slices * M * rows * (long)sizeof(float);
+  FMS_REQUIRE(workspace != nullptr && workspace_bytes >= needed, "wide product: workspace of %ld bytes, %ld needed",
+              workspace_bytes, needed);
   dim3 grid(ceil_div(rows, WD_ROWS), slices);
   FMS_REQUIRE(grid.y <= 65535, "wide product: %d slices", slices);
   float* part = (float*)workspace;
-  const int mt = ceil_div(M, 16);
-  if (mt == 2)
-    wide_partial_kernel<2><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice);
-  else if (mt == 3)
-    wide_partial_kernel<3><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice);
-  else
-    wide_partial_kernel<4><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice);
+  o.vec = aligned16(workspace) && rows % 4 == 0;
+  launch_wide<WD_PARTIAL, float>(grid, x, ldx, w, part, M, rows, K, per_slice, o, stream);
   FMS_LAUNCH_CHECK("wide product");
   switch (epi) {
     case EPI_PLAIN:

@@ -331,7 +331,7 @@ def test_gemm_f32(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 48, 64, 65, 200, 300])
-@pytest.mark.parametrize("N,K", [(40, 24), (100, 176), (384, 96), (4096 + 16, 512), (20000, 64)])
+@pytest.mark.parametrize("N,K", [(40, 24), (100, 176), (257, 96), (384, 96), (4096 + 16, 512), (20000, 64)])
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(7)
     x = torch.randn(M, K).to(torch.bfloat16)
@@ -354,7 +354,7 @@ def test_gemm_bf16(ops, M, N, K):
 
 
 @pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100])
-@pytest.mark.parametrize("hidden,K", [(44, 24), (176, 64), (1000, 96)])
+@pytest.mark.parametrize("hidden,K", [(44, 24), (77, 40), (176, 64), (1000, 96)])
 def test_gated_linear(ops, M, hidden, K):
     torch.manual_seed(8)
     for dtype in (torch.bfloat16, torch.float32):
