@@ -628,23 +628,33 @@ __device__ __forceinline__ void decode_keys(WaveState<MAXDT, 1>& st, const bf16x
   decode_math<MAXDT, HALVES>(st, qreg, qpos, qlo, key0, kreg, vreg, head_dim, scale2);
 }
 
-// A whole page of head size 128 by way of the wave's own 16 KB of LDS.  The page of a kv head is 16 KB of
-// keys and 16 KB of values, each contiguous: the wave loads them 1 KB an instruction (what the memory system
-// streams best; the operand layout takes 64 bytes from each of 16 rows and fetches every line twice), writes
-// them to LDS as loaded and reads the MFMA operands back: first the keys, then, through the same buffer, the
-// values.  16-byte pieces are XOR-swizzled so that both directions spread over the banks.
-__device__ __forceinline__ void decode_page_staged(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
-                                                   int key0, const bf16* __restrict__ kp, const bf16* __restrict__ vp,
-                                                   bf16* __restrict__ buf, float scale2) {
+// Pages of head size 128 by way of the wave's own 16 KB of LDS.  The page of a kv head is 16 KB of keys and
+// 16 KB of values, each contiguous: the wave loads them 1 KB an instruction (what the memory system streams
+// best; the operand layout takes 64 bytes from each of 16 rows and fetches every line twice), writes them to
+// LDS as loaded and reads the MFMA operands back: first the keys, then, through the same buffer, the values.
+// 16-byte pieces are XOR-swizzled so that both directions spread over the banks.
+//
+// The wave's pages are a pipeline through one set of 16 load registers: as soon as the keys of a page are in
+// LDS the registers take the loads of its values, and as soon as those are in LDS, the loads of the next
+// page's keys; so the memory always works on the wave's next 16 KB while the matrix unit works on the last.
+// A compute unit's loads queue up behind one another (16 KB asked for when the unit's other waves have just
+// asked for theirs take some microseconds); a wave that asks again the moment its registers are free keeps
+// that queue full instead of waiting at its end once a page.
+__device__ __forceinline__ void staged_load(bf16x8 (&raw)[16], const bf16* __restrict__ p) {
+  const int lane = threadIdx.x & (WAVE - 1);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) raw[i] = load_bf16x8(p + i * 512 + lane * 8);
+}
+
+// One page: its keys are on their way into raw; vp points at its values, kn (PREFETCH) at the next page's
+// keys.  The softmax takes the page's 64 keys at once.
+template <bool PREFETCH>
+__device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
+                                                 int key0, bf16x8 (&raw)[16], const bf16* __restrict__ vp,
+                                                 const bf16* __restrict__ kn, bf16* __restrict__ buf, float scale2) {
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15;
   const int g = lane >> 4;
-  bf16x8 kraw[16], vraw[16];
-#pragma unroll
-  for (int i = 0; i < 16; ++i) kraw[i] = load_bf16x8(kp + i * 512 + lane * 8);
-#pragma unroll
-  for (int i = 0; i < 16; ++i) vraw[i] = load_bf16x8(vp + i * 512 + lane * 8);
-
   // keys: row = token (256 bytes = 16 pieces), piece ^ key(token); the 16 tokens of a score tile have the keys 0..15
   {
     const int piece = lane & 15;
@@ -652,39 +662,120 @@ __device__ __forceinline__ void decode_page_staged(WaveState<8, 1>& st, const bf
     for (int i = 0; i < 16; ++i) {
       const int token = i * 4 + (lane >> 4);
       const int key = (((token >> 3) & 3) << 2) | (token & 3);
-      *reinterpret_cast<bf16x8*>(buf + token * 128 + ((piece ^ key) & 15) * 8) = kraw[i];
+      *reinterpret_cast<bf16x8*>(buf + token * 128 + ((piece ^ key) & 15) * 8) = raw[i];
     }
   }
   __builtin_amdgcn_wave_barrier();
-  bf16x8 kreg[2][2][4], vreg[2][8];
-  const int key_a = (r >> 2) * 8 + (r & 3);  // its swizzle key is r, and so is that of key_a + 4
+  staged_load(raw, vp);
+  // Which key sits in which row of the two score tiles: see decode_keys.  The swizzle key of row key_a is r,
+  // and so is that of key_a + 4.
+  const int key_a = (r >> 2) * 8 + (r & 3);
+  f32x4 sa[2], sb[2];
 #pragma unroll
-  for (int hf = 0; hf < 2; ++hf)
+  for (int hf = 0; hf < 2; ++hf) {
+    bf16x8 ka[4], kb[4];
 #pragma unroll
-    for (int tile = 0; tile < 2; ++tile)
+    for (int c = 0; c < 4; ++c) {
+      ka[c] = *reinterpret_cast<const bf16x8*>(buf + (hf * 32 + key_a) * 128 + (((c * 4 + g) ^ r) & 15) * 8);
+      kb[c] = *reinterpret_cast<const bf16x8*>(buf + (hf * 32 + key_a + 4) * 128 + (((c * 4 + g) ^ r) & 15) * 8);
+    }
+    sa[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
+    sb[hf] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int c = 0; c < 4; ++c)
-        kreg[hf][tile][c] = *reinterpret_cast<const bf16x8*>(buf + (hf * 32 + key_a + 4 * tile) * 128 + (((c * 4 + g) ^ r) & 15) * 8);
-  __builtin_amdgcn_wave_barrier();
+    for (int c = 0; c < 4; ++c) {
+      sa[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[c], qreg[c], sa[hf], 0, 0, 0);
+      sb[hf] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[c], qreg[c], sb[hf], 0, 0, 0);
+    }
+  }
+
+  float mx = -INFINITY;
+  if (key0 + PAGE_TOKENS - 1 <= qpos && key0 >= qlo) {  // uniform: all 64 keys are visible
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(sa[hf][i], sb[hf][i]));
+  } else {
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int ja = key0 + hf * 32 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
+        const int jb = ja + 4;
+        sa[hf][i] = (ja <= qpos && ja >= qlo) ? sa[hf][i] : -INFINITY;
+        sb[hf][i] = (jb <= qpos && jb >= qlo) ? sb[hf][i] : -INFINITY;
+        mx = fmaxf(mx, fmaxf(sa[hf][i], sb[hf][i]));
+      }
+  }
+  mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
+  mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+  const float m_new = fmaxf(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
+  const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
+  st.m[0] = m_new;
+  bf16x8 pmat[2];
+  float psum = 0.f;
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    float pa[4], pb[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      pa[i] = __builtin_amdgcn_exp2f(fmaf(sa[hf][i], scale2, -m_new));
+      pb[i] = __builtin_amdgcn_exp2f(fmaf(sb[hf][i], scale2, -m_new));
+      psum += pa[i] + pb[i];
+    }
+    pmat[hf] = bf16x8{(bf16)pa[0], (bf16)pa[1], (bf16)pa[2], (bf16)pa[3], (bf16)pb[0], (bf16)pb[1], (bf16)pb[2], (bf16)pb[3]};
+  }
+  st.l[0] = st.l[0] * alpha + psum;
+  if (__any(alpha != 1.f)) {  // the running maximum seldom moves after the first keys
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) st.acc[0][dt] *= alpha;
+  }
+
+  __builtin_amdgcn_wave_barrier();  // the keys have been read: the buffer takes the values
   // values: row = d (128 bytes = 8 pieces of 8 tokens), piece ^ (d / 2): two rows fill the banks once
   {
     const int piece = lane & 7;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int d = i * 8 + (lane >> 3);
-      *reinterpret_cast<bf16x8*>(buf + d * 64 + ((piece ^ (d >> 1)) & 7) * 8) = vraw[i];
+      *reinterpret_cast<bf16x8*>(buf + d * 64 + ((piece ^ (d >> 1)) & 7) * 8) = raw[i];
     }
   }
   __builtin_amdgcn_wave_barrier();
+  if (PREFETCH) staged_load(raw, kn);
 #pragma unroll
-  for (int hf = 0; hf < 2; ++hf)
+  for (int hf = 0; hf < 2; ++hf) {
+    bf16x8 vreg[8];
 #pragma unroll
     for (int dt = 0; dt < 8; ++dt) {
       const int d = dt * 16 + r;
-      vreg[hf][dt] = *reinterpret_cast<const bf16x8*>(buf + d * 64 + (((hf * 4 + g) ^ (d >> 1)) & 7) * 8);
+      vreg[dt] = *reinterpret_cast<const bf16x8*>(buf + d * 64 + (((hf * 4 + g) ^ (d >> 1)) & 7) * 8);
     }
-  __builtin_amdgcn_wave_barrier();
-  decode_math<8, 2>(st, qreg, qpos, qlo, key0, kreg, vreg, 128, scale2);
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt)
+      st.acc[0][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vreg[dt], pmat[hf], st.acc[0][dt], 0, 0, 0);
+  }
+  __builtin_amdgcn_wave_barrier();  // the values have been read: the buffer is free for the next page's keys
+}
+
+// The pages first, first + stride, ... <= last of a sequence, for kv head kh.
+__device__ __forceinline__ void decode_pages_staged(WaveState<8, 1>& st, const bf16x8 (&qreg)[4], int qpos, int qlo,
+                                                    int first, int stride, int last, const int* __restrict__ bt,
+                                                    const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache,
+                                                    size_t page_elems, int kh, bf16* __restrict__ buf, float scale2) {
+  if (first > last) return;
+  const size_t head_off = (size_t)kh * PAGE_TOKENS * 128;
+  bf16x8 raw[16];
+  size_t phys = (size_t)uniform_load(bt + first);
+  staged_load(raw, k_cache + phys * page_elems + head_off);
+  int pi = first;
+  for (; pi + stride <= last; pi += stride) {
+    const size_t next = (size_t)uniform_load(bt + pi + stride);
+    staged_page_step<true>(st, qreg, qpos, qlo, pi * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off,
+                           k_cache + next * page_elems + head_off, buf, scale2);
+    phys = next;
+  }
+  staged_page_step<false>(st, qreg, qpos, qlo, pi * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off, nullptr,
+                          buf, scale2);
 }
 
 // The pages that split `split` of `n_splits` takes of a sequence whose visible keys are lo..pos: every
@@ -711,7 +802,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
                             const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                             const int* __restrict__ block_table, int table_stride, const bf16* __restrict__ k_cache,
                             const bf16* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale,
-                            int window, int tile_cols) {
+                            int window, int tile_cols, const int* __restrict__ row_order) {
   extern __shared__ float lds_dynamic[];  // not staged: [wave][tile_cols columns][head_dim + 2]
   __shared__ __attribute__((aligned(16))) bf16 stage[STAGED ? MAXW * 8192 : 8];
   // where the waves' partial results meet: a region of its own, or (staged) the head of each wave's page buffer
@@ -722,7 +813,8 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   const int tiles_per_kv = (group + tile_cols - 1) / tile_cols;
   const int kh = blockIdx.y / tiles_per_kv;
   const int ht = blockIdx.y % tiles_per_kv;
-  const int t = blockIdx.z;
+  // blocks are handed out in the order of their index: with the rows sorted by length the long ones go first
+  const int t = row_order != nullptr ? uniform_load(row_order + blockIdx.z) : (int)blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);  // uniform: table entries load as scalars
   const int n_waves = blockDim.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
@@ -750,18 +842,21 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
 
   WaveState<MAXDT, 1> st;
   wave_state_init(st);
-  for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
-    const size_t phys = (size_t)uniform_load(bt + pi);
-    const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
-    const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
-    if (STAGED) {
-      if constexpr (MAXDT == 8)
-        decode_page_staged(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, stage + wave * 8192, scale * LOG2E);
-    } else if (MAXDT <= 8) {
-      decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
-    } else {  // large heads: half a page at a time keeps the loads in registers
-      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
-      decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, scale * LOG2E);
+  if (STAGED) {
+    if constexpr (MAXDT == 8)
+      decode_pages_staged(st, qreg, pos, lo, page_lo + wave, n_waves, page_hi, bt, k_cache, v_cache, page_elems, kh,
+                          stage + wave * 8192, scale * LOG2E);
+  } else {
+    for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
+      const size_t phys = (size_t)uniform_load(bt + pi);
+      const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
+      const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
+      if (MAXDT <= 8) {
+        decode_keys<MAXDT, 2>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
+      } else {  // large heads: half a page at a time keeps the loads in registers
+        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS, kp, vp, head_dim, scale * LOG2E);
+        decode_keys<MAXDT, 1>(st, qreg, pos, lo, pi * PAGE_TOKENS + 32, kp, vp, head_dim, scale * LOG2E);
+      }
     }
   }
 
@@ -957,7 +1052,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
                                        const int* block_table, int table_stride, const void* k_cache,
                                        const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim,
                                        float scale, int window, int max_context, int pages_per_split, int waves,
-                                       int staged, hipStream_t stream) {
+                                       int staged, const int* row_order, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (check_common("attn_decode_bf16", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(head_dim % 16 == 0, "attn_decode_bf16: head size %d is no multiple of 16", head_dim);
@@ -984,7 +1079,7 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   attn_decode_bf16_kernel<M, MAXW, STAGED><<<grid, dim3(waves * WAVE), LDS, stream>>>(                               \
       (const bf16*)q, q_stride, (bf16*)out, out_stride, part_o, part_ml, n_splits, positions, seq_of_token,          \
       block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale,       \
-      window, tile_cols)
+      window, tile_cols, row_order)
   FMS_REQUIRE(staged == 0 || head_dim == 128, "attn_decode_bf16: pages go through LDS for head size 128 only");
   if (staged != 0) {
     // the waves' results meet in the page buffers: 16 KB a wave hold 16 columns of 130 floats

@@ -74,13 +74,15 @@ int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out, long out_s
 // `pages_per_split` pages, and every sequence deals its own pages out evenly over that many blocks of `waves`
 // waves (which take them in turn and merge in LDS); with more than one split a second kernel merges the
 // partial results.  staged != 0 (head size 128 only): pages are loaded in contiguous kilobytes and turned into
-// the MFMA layout in LDS, which streams faster when there is much to read.
+// the MFMA layout in LDS, which streams faster when there is much to read.  row_order (or null): the token rows in
+// the order in which the blocks are to take them, e.g. longest context first; the result does not depend on it.
 long fmsamd_attn_decode_workspace(int n_tokens, int nheads, int head_dim, int n_splits);
 int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, long out_stride, void* workspace,
                             long workspace_bytes, const int* positions, const int* seq_of_token,
                             const int* block_table, int table_stride, const void* k_cache, const void* v_cache,
                             int n_tokens, int nheads, int kvheads, int head_dim, float scale, int window,
-                            int max_context, int pages_per_split, int waves, int staged, hipStream_t stream);
+                            int max_context, int pages_per_split, int waves, int staged, const int* row_order,
+                            hipStream_t stream);
 
 // c[M, N] = a[M, K] w[N, K]^T (+ bias[N])
 int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias, float* c, long ldc, int M, int N,

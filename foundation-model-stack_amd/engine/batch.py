@@ -32,6 +32,9 @@ class StepBatch:
     qblocks: Dict[int, tuple] = dataclasses.field(default_factory=dict)
     logit_rows: Optional[torch.Tensor] = None  # int32 [n_wanted] token indices whose logits are wanted
     n_logit_rows: int = 0
+    # decode steps: the token rows from the longest context to the shortest (int32 [T]).  A kernel whose blocks
+    # take a sequence each hands out the long ones first, so that none of them is left to run alone at the end.
+    rows_by_length: Optional[torch.Tensor] = None
 
 
 def build_batch(
@@ -73,7 +76,9 @@ def build_batch(
     tables = {g: cache.block_table(g, slots) for g in range(len(cache.groups))}
 
     # one host buffer, one copy
-    parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows]
+    is_decode = all(n == 1 for n in q_lens)
+    by_length = sorted(range(T), key=lambda t: -positions[t]) if is_decode else []
+    parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows, by_length]
     for size in sizes:
         parts += [qb_start[size], qb_len[size]]
     lengths = [len(p) for p in parts]
@@ -104,7 +109,7 @@ def build_batch(
         slots=list(slots),
         q_lens=q_lens,
         starts=list(starts),
-        is_decode=all(n == 1 for n in q_lens),
+        is_decode=is_decode,
         max_context=max(s + n for s, n in zip(starts, q_lens)),
         context_bound=max(s + n for s, n in zip(starts, q_lens)),
         token_ids=span(0),
@@ -113,7 +118,8 @@ def build_batch(
         slot_ids=span(3),
         seq_starts=span(4),
         block_tables={g: dev[o : o + shape[0] * shape[1]].view(shape) for g, (o, shape) in table_spans.items()},
-        qblocks={size: (span(6 + 2 * i), span(7 + 2 * i)) for i, size in enumerate(sizes)},
+        qblocks={size: (span(7 + 2 * i), span(8 + 2 * i)) for i, size in enumerate(sizes)},
         logit_rows=span(5),
         n_logit_rows=len(rows),
+        rows_by_length=span(6) if is_decode else None,
     )

@@ -59,13 +59,14 @@ class DecodeGraph:
         self.slot_ids = torch.zeros(rows, dtype=torch.int32, device=dev)
         self.seq_starts = torch.arange(rows + 1, dtype=torch.int32, device=dev)
         self.logit_rows = torch.arange(rows, dtype=torch.int32, device=dev)
+        self.rows_by_length = torch.arange(rows, dtype=torch.int32, device=dev)
         self.tables = {g: torch.zeros(rows, self.table_width, dtype=torch.int32, device=dev) for g in range(len(cache.groups))}
         self.rng = torch.zeros(rows, 2, dtype=torch.int64, device=dev)
         self.batch = StepBatch(
             n_tokens=rows, n_seqs=rows, slots=[], q_lens=[1] * rows, starts=[0] * rows, is_decode=True,
             max_context=max_context, context_bound=max_context, token_ids=self.tokens, positions=self.positions, seq_of_token=self.seq_of_token,
             slot_ids=self.slot_ids, seq_starts=self.seq_starts, block_tables=self.tables,
-            logit_rows=self.logit_rows, n_logit_rows=rows,
+            logit_rows=self.logit_rows, n_logit_rows=rows, rows_by_length=self.rows_by_length,
         )
         # what the static buffers currently describe
         self.slots: Tuple[int, ...] = ()
@@ -114,6 +115,9 @@ class DecodeGraph:
         self.positions.copy_(torch.tensor(list(positions) + [0] * pad, dtype=torch.int32), non_blocking=True)
         self.seq_of_token.copy_(torch.tensor(list(range(n)) + [-1] * pad, dtype=torch.int32), non_blocking=True)
         self.slot_ids.copy_(torch.tensor(list(slots) + [0] * pad, dtype=torch.int32), non_blocking=True)
+        # every sequence grows by one token a step: the order of the lengths holds as long as the batch does
+        order = sorted(range(n), key=lambda b: -positions[b]) + list(range(n, self.rows))
+        self.rows_by_length.copy_(torch.tensor(order, dtype=torch.int32), non_blocking=True)
         for g, table in self.tables.items():
             host = cache.block_table(g, slots, n_columns=self.table_width)
             table[:n].copy_(host, non_blocking=True)

@@ -35,7 +35,7 @@ _SIGNATURES = {
     "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, P],
     "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, P],
-    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P],
+    "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, P],
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
     "fmsamd_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],

@@ -334,12 +334,14 @@ def attention(
     waves: int = 0,
     force_generic: bool = False,
     staged: Optional[bool] = None,
+    row_order: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim].
 
     q is a [T, >= nheads*head_dim] view (the query columns of the qkv rows).  float32 runs the
     generic kernel; bfloat16 runs the MFMA kernels (prefill needs the query blocks, decode the
-    largest context).
+    largest context).  row_order (decode, optional): int32 [T], the token rows in the order in which the
+    kernel's blocks are to take them, longest context first; the result does not depend on it.
     """
     _need_cuda(q, positions, seq_of_token, block_table, k_cache, v_cache)
     _rows2d("q", q)
@@ -366,13 +368,18 @@ def attention(
         if waves <= 0:
             waves = min(auto_waves, pages_per_block)
         n_splits = -(-n_pages // pages_per_block)
+        if row_order is not None:
+            _need_cuda(row_order)
+            _need_i32("row_order", row_order)
+            if row_order.numel() != T or not row_order.is_contiguous():
+                raise ValueError(f"row_order has {row_order.numel()} entries for {T} tokens")
         ws_bytes = lib.fmsamd_attn_decode_workspace(T, nheads, head_dim, n_splits)
         ws = torch.empty(max(ws_bytes // 4, 1), dtype=torch.float32, device=q.device) if ws_bytes else None
         check(lib.fmsamd_attn_decode_bf16(q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), _ptr(ws), ws_bytes,
                                           positions.data_ptr(), seq_of_token.data_ptr(), block_table.data_ptr(),
                                           block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), T, nheads, kvheads,
                                           head_dim, float(scale), int(window), int(max_context), int(pages_per_block), int(waves),
-                                          int(bool(staged)) if staged is not None else int(head_dim == 128), _stream()))
+                                          int(bool(staged)) if staged is not None else int(head_dim == 128), _ptr(row_order), _stream()))
         return out
     if qblock_start is None or qblock_len is None:
         raise ValueError("bfloat16 prefill attention needs the query blocks of the batch")
@@ -390,12 +397,12 @@ def decode_split(rows: int, n_pages: int):
 
     rows = tokens x kv heads.  A compute unit pulls only a small share of the memory bandwidth, so
     the cache has to be spread over all of them: the context bound is cut into as many splits as give
-    a few hundred blocks, and at least so many that a block has no more than 16 pages (every sequence
-    deals its own pages out evenly over the splits, so a long sequence among short ones does not end
-    up in one block).  The waves of a block share its pages and merge in LDS, the blocks of a row
+    a few hundred blocks, and at least so many that a block has no more than 128 pages (every sequence
+    deals its own pages out evenly over the splits; the waves of a block run their pages as a pipeline,
+    so a block of many pages is cheaper than many blocks).  The waves of a block share its pages and merge in LDS, the blocks of a row
     merge in a second kernel."""
-    by_rows = min(-(-256 // max(rows, 1)), max(1, n_pages // 4))  # but no splits of under 4 pages
-    splits = max(1, min(max(by_rows, -(-n_pages // 16)), n_pages))
+    by_rows = min(-(-256 // max(rows, 1)), max(1, n_pages // 8))  # but no splits of under 8 pages: one for each wave
+    splits = max(1, min(max(by_rows, -(-n_pages // 128)), n_pages))
     pages = -(-n_pages // splits)
     waves = max(1, min(8 if rows * splits <= 512 else 4, pages))
     return pages, waves

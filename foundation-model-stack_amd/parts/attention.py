@@ -107,6 +107,7 @@ class MultiHeadAttention(Mixer):
             qkv, batch.positions, batch.seq_of_token, table, cache.keys, cache.values, H, K, D, self.scale, self.window,
             decode=batch.is_decode, max_context=batch.context_bound,
             qblock_start=qb_start, qblock_len=qb_len, qblock_tokens=size,
+            row_order=batch.rows_by_length if batch.is_decode else None,
         )
         return BranchOutput(mixed, self.dense)
 

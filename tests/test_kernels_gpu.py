@@ -298,6 +298,9 @@ def test_attention_decode_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=5, waves=3)
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=24, waves=8)
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2, 600], lens=[1, 1, 1], decode=True, pages_per_block=16, waves=4)
+    # the order in which the blocks take the rows changes nothing; several pages a wave run as a pipeline
+    attention_case(ops, torch.bfloat16, H, K, D, starts=[40, 1500, 2, 600], lens=[1, 1, 1, 1], decode=True, pages_per_block=24, waves=2,
+                   row_order=dev(torch.tensor([1, 3, 0, 2], dtype=torch.int32)))
     if D == 128:
         # pages by way of LDS: blocks of up to 4 and of up to 8 waves, whole and partly filled pages, splits
         for pages, waves in ((64, 8), (64, 3), (5, 2), (2, 1), (16, 4)):
