@@ -301,3 +301,136 @@ def test_a_layer_named_twice_and_a_layer_reading_another_cache(lib, tmp_path):
     slot = engine.new_sequence()
     got = [engine.step([slot], [ids[:70]], "all")] + [engine.step([slot], [[t]], "last") for t in ids[70:]]
     torch.testing.assert_close(torch.cat(got).cpu(), plain(ids), atol=2e-4, rtol=1e-3)
+
+
+def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(lib):
+    """Two more kinds of part that the library does not have, defined here and registered by name:
+    a feed-forward that routes every token to one of three small experts (router logits and the chosen
+    expert's probability in float32), and a position encoding that is no rotation (queries grow and keys
+    shrink geometrically with the position, so a score is damped by the distance between them).
+    One layer uses both, the other the library's own feed-forward; the model is built by get_model,
+    stepped by Engine (prompts whole, then token by token, two sequences of unequal length) and
+    compared with a plain computation that knows nothing of the parts."""
+    import fms_amd
+    from fms_amd.architectures import Architecture, register_architecture, register_model
+    from fms_amd.config import ModelConfig
+    from fms_amd.engine import Engine
+    from fms_amd.engine.model import DecoderModel
+    from fms_amd.weights import init_random
+    from fms_amd.parts import FeedForward, LayerSpec, ModelSpec, PartSpec, register_part, unregister_part
+    from fms_amd.parts.position import PositionEncoding
+
+    class RoutedFeedForward(FeedForward):
+        def __init__(self, width, hidden_dim, n_experts):
+            super().__init__()
+            self.width, self.hidden, self.n = width, hidden_dim, n_experts
+            self.declare("router.weight", (n_experts, width))
+            self.declare("experts.up", (n_experts, hidden_dim, width))
+            self.declare("experts.down", (n_experts, width, hidden_dim))
+
+        def forward(self, x):
+            xf = x.float()
+            logits = xf @ self.w["router.weight"].float().t()
+            prob = torch.softmax(logits, -1)
+            choice = logits.argmax(-1)
+            out = torch.zeros_like(xf)
+            for e in range(self.n):  # every expert on every token, the unchosen ones times zero: no host decision
+                y = torch.relu(xf @ self.w["experts.up"][e].float().t()) @ self.w["experts.down"][e].float().t()
+                out += y * (prob[:, e] * (choice == e))[:, None]
+            return out.to(x.dtype)
+
+    class DistanceDamping(PositionEncoding):
+        def __init__(self, rate):
+            super().__init__()
+            self.rate = float(rate)
+
+        def adjust_qk(self, qkv, batch, nheads, kvheads, head_dim):
+            grow = torch.pow(torch.tensor(self.rate, device=qkv.device), -batch.positions.float())[:, None]
+            q_cols, k_cols = nheads * head_dim, kvheads * head_dim
+            qkv[:, :q_cols] = (qkv[:, :q_cols].float() / grow).to(qkv.dtype)  # q_i * rate^i
+            qkv[:, q_cols : q_cols + k_cols] = (qkv[:, q_cols : q_cols + k_cols].float() * grow).to(qkv.dtype)  # k_j * rate^-j
+
+    @dataclasses.dataclass
+    class ToyConfig(ModelConfig):
+        vocab: int = 77
+        width: int = 40
+        hidden: int = 56
+        max_len: int = 128
+
+    H, K, D, RATE = 5, 1, 8, 0.97
+
+    def toy_spec(c: ToyConfig) -> ModelSpec:
+        norm = PartSpec("rmsnorm", {"eps": 1e-6})
+        attn = PartSpec("attention", {"nheads": H, "kvheads": K, "head_dim": D})
+        routed = LayerSpec(mixer=attn, feed_forward=PartSpec("routed", {"hidden_dim": 24, "n_experts": 3}), norm=norm, position="damp")
+        dense = LayerSpec(mixer=attn, feed_forward=PartSpec("glu", {"hidden_dim": c.hidden, "activation": "swish"}), norm=norm,
+                          position="damp")
+        return ModelSpec(vocab=c.vocab, width=c.width, max_seq_len=c.max_len, layers=[routed, dense], final_norm=norm,
+                         positions={"damp": PartSpec("distance_damping", {"rate": RATE})})
+
+    register_part("feed_forward", "routed", RoutedFeedForward)
+    register_part("position", "distance_damping", DistanceDamping)
+    try:
+        try:
+            register_architecture(Architecture("toy_routed", ToyConfig, toy_spec))
+            register_model("toy_routed", "tiny", lambda **kw: ToyConfig().updated(**kw))
+        except KeyError:
+            pass  # a second run in one process
+        built = fms_amd.get_model("toy_routed", "tiny", data_type="float32", random_seed=4)
+        assert isinstance(built.layers[0].feed_forward, RoutedFeedForward) and isinstance(built.positions["damp"], DistanceDamping)
+        # weights of std 0.02 would leave the router undecided and the damping invisible: the same model, wider weights
+        model = DecoderModel(toy_spec(ToyConfig()), torch.float32, config=ToyConfig())
+        init_random(model, 4, torch.device(DEV), std=0.2, norm_std=0.1)
+        model.finalize_all(DEV)
+        engine = Engine(model, max_tokens=256, max_slots=2)
+        w = {name: owner.w[local].float().cpu() for name, _, owner, local in model.named_specs()}
+
+        def plain(ids):
+            S = len(ids)
+            x = w["base_model.embedding.weight"][torch.tensor(ids)]
+            dist = torch.arange(S)[:, None] - torch.arange(S)[None, :]
+            damp = torch.where(dist >= 0, RATE ** dist.clamp(min=0).float(), torch.zeros(()))
+            for layer in (0, 1):
+                p = f"base_model.layers.{layer}."
+                h = P.rms_norm(x, w[p + "ln.weight"], 1e-6)
+                q, k, v = torch.split(h @ w[p + "attn.in_proj.qkv_fused.weight"].t(), [H * D, K * D, K * D], dim=-1)
+                q, k, v = q.reshape(S, H, D), k.reshape(S, K, D), v.reshape(S, K, D)
+                scores = torch.einsum("ihd,jd->hij", q, k[:, 0]) * damp / math.sqrt(D)
+                scores = scores.masked_fill(dist < 0, float("-inf"))
+                mixed = torch.einsum("hij,jd->ihd", torch.softmax(scores, -1), v[:, 0]).reshape(S, H * D)
+                x = x + mixed @ w[p + "attn.dense.weight"].t()
+                h = P.rms_norm(x, w[p + "ff_ln.weight"], 1e-6)
+                if layer == 0:
+                    logits = h @ w[p + "ff_sub_layer.router.weight"].t()
+                    choice = logits.argmax(-1)
+                    prob = torch.softmax(logits, -1)[torch.arange(S), choice]
+                    up, down = w[p + "ff_sub_layer.experts.up"][choice], w[p + "ff_sub_layer.experts.down"][choice]
+                    y = torch.einsum("sdh,sh->sd", down, torch.relu(torch.einsum("shd,sd->sh", up, h)))
+                    x = x + y * prob[:, None]
+                else:
+                    x = x + P.gated_feed_forward(h, w[p + "ff_sub_layer.wg1_fused.weight"], w[p + "ff_sub_layer.w2.weight"])
+            return P.rms_norm(x, w["base_model.dec_norm.weight"], 1e-6) @ w["head.weight"].t()
+
+        g = torch.Generator().manual_seed(2)
+        seqs = [torch.randint(0, 77, (n,), generator=g).tolist() for n in (41, 12)]
+        slots = [engine.new_sequence() for _ in seqs]
+        got = [[], []]
+        logits = engine.step(slots, [s[:-3] for s in seqs], "all")
+        got[0].append(logits[: len(seqs[0]) - 3])
+        got[1].append(logits[len(seqs[0]) - 3 :])
+        for i in range(3, 0, -1):
+            logits = engine.step(slots, [[s[-i]] for s in seqs], "last")
+            got[0].append(logits[0:1])
+            got[1].append(logits[1:2])
+        for ids, rows in zip(seqs, got):
+            torch.testing.assert_close(torch.cat(rows).cpu(), plain(ids), atol=2e-4, rtol=1e-3)
+        # and the damping did something: without it the logits differ visibly
+        RATE_KEEP = RATE
+        try:
+            RATE = 1.0
+            assert (plain(seqs[0]) - torch.cat(got[0]).cpu()).abs().max() > 1e-3
+        finally:
+            RATE = RATE_KEEP
+    finally:
+        unregister_part("feed_forward", "routed")
+        unregister_part("position", "distance_damping")
