@@ -31,7 +31,8 @@ extern "C" int fmsamd_rope_table(const float* freqs, float* cos_t, float* sin_t,
   return 0;
 }
 
-// One block per token.  qkv row = [H*D queries | K*D keys | K*D values].
+// One block per token, a pair of elements a thread: for any even head size and any alignment.
+// qkv row = [H*D queries | K*D keys | K*D values].
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
                                      const int* __restrict__ seq_of_token, const int* __restrict__ block_table,
@@ -85,6 +86,98 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const
   }
 }
 
+// The same for many tokens: a block takes RT consecutive token rows and one head (a query head, a key head or
+// a value head), four elements a thread.  Rows of q and k stay rows; the values of a head are turned over in
+// LDS, so that the lanes of a store are neighbouring tokens of one row of the transposed page (tokens that
+// follow one another in a sequence are neighbours there) instead of 2-byte writes 128 bytes apart.
+template <typename T>
+struct Vec4 {
+  typedef T type __attribute__((ext_vector_type(4)));
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+    rope_kv_tile_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
+                        const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
+                        const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot_dim, int max_pos,
+                        T* __restrict__ k_cache, T* __restrict__ v_cache, int nheads, int kvheads, int head_dim,
+                        int n_tokens) {
+  constexpr int RT = sizeof(T) == 4 ? 32 : 64;
+  typedef typename Vec4<T>::type vec4;
+  extern __shared__ __attribute__((aligned(16))) unsigned char tile_raw[];  // value heads: RT x (head_dim + 4)
+  __shared__ int s_pos[RT];
+  __shared__ long long s_page[RT];  // -1: the row is padding or past the end
+  const int t0 = blockIdx.x * RT;
+  const int hh = blockIdx.y;
+  if (hh >= nheads && k_cache == nullptr) return;  // queries only
+  if (threadIdx.x < RT) {
+    const int t = t0 + threadIdx.x;
+    int pos = 0;
+    long long page = -1;
+    if (t < n_tokens) {
+      const int seq = seq_of_token[t];
+      if (seq >= 0) {
+        pos = positions[t];
+        page = k_cache ? block_table[(size_t)seq * table_stride + pos / PAGE_TOKENS] : 0;
+      }
+    }
+    s_pos[threadIdx.x] = pos;
+    s_page[threadIdx.x] = page;
+  }
+  __syncthreads();
+  const int quads = head_dim / 4;
+  const int rot_half = rot_dim / 2;
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  if (hh < nheads + kvheads) {
+    for (int idx = threadIdx.x; idx < RT * quads; idx += blockDim.x) {
+      const int tok = idx / quads, qd = idx - tok * quads;
+      if (s_page[tok] < 0) continue;
+      const int pos = s_pos[tok];
+      T* p = qkv + (size_t)(t0 + tok) * row_stride + (size_t)hh * head_dim + 4 * qd;
+      vec4 v = *reinterpret_cast<const vec4*>(p);
+      if (cos_t != nullptr) {
+        const int tpos = pos < max_pos ? pos : max_pos - 1;  // the host has checked; never read outside the table
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          const int i = 2 * qd + j;  // the pair (x[2i], x[2i+1])
+          if (i < rot_half) {
+            const float c = cos_t[(size_t)tpos * rot_half + i];
+            const float sn = sin_t[(size_t)tpos * rot_half + i];
+            const float a = to_f32(v[2 * j]), b = to_f32(v[2 * j + 1]);
+            v[2 * j] = from_f32<T>(c * a - sn * b);
+            v[2 * j + 1] = from_f32<T>(sn * a + c * b);
+          }
+        }
+      }
+      if (hh < nheads) {
+        *reinterpret_cast<vec4*>(p) = v;
+      } else {
+        const int kh = hh - nheads;
+        T* dst = k_cache + (size_t)s_page[tok] * page_elems + ((size_t)kh * PAGE_TOKENS + pos % PAGE_TOKENS) * head_dim + 4 * qd;
+        *reinterpret_cast<vec4*>(dst) = v;
+      }
+    }
+    return;
+  }
+
+  T* tile = reinterpret_cast<T*>(tile_raw);
+  const int ld = head_dim + 4;
+  for (int idx = threadIdx.x; idx < RT * quads; idx += blockDim.x) {
+    const int tok = idx / quads, qd = idx - tok * quads;
+    if (s_page[tok] < 0) continue;
+    *reinterpret_cast<vec4*>(tile + tok * ld + 4 * qd) =
+        *reinterpret_cast<const vec4*>(qkv + (size_t)(t0 + tok) * row_stride + (size_t)hh * head_dim + 4 * qd);
+  }
+  __syncthreads();
+  const int kh = hh - nheads - kvheads;
+  for (int idx = threadIdx.x; idx < RT * head_dim; idx += blockDim.x) {
+    const int tok = idx % RT, d = idx / RT;  // neighbouring lanes: neighbouring tokens
+    if (s_page[tok] < 0) continue;
+    v_cache[(size_t)s_page[tok] * page_elems + ((size_t)kh * head_dim + d) * PAGE_TOKENS + s_pos[tok] % PAGE_TOKENS] = tile[tok * ld + d];
+  }
+}
+
 extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* positions,
                                     const int* seq_of_token, const int* block_table, int table_stride,
                                     const float* cos_t, const float* sin_t, int rot_dim, int max_pos, void* k_cache,
@@ -100,16 +193,32 @@ extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const
   FMS_REQUIRE(cos_t == nullptr || max_pos > 0, "rope_kv_write: empty table");
   const int threads = 256;
   const float* c = rot_dim > 0 ? cos_t : nullptr;
-  if (dtype == FMS_F32)
+  const size_t elem = dtype == FMS_F32 ? 4 : 2;
+  FMS_REQUIRE(dtype == FMS_F32 || dtype == FMS_BF16, "rope_kv_write: unknown dtype %d", dtype);
+  // four elements a thread need rows that start at multiples of four elements
+  const bool by_fours = head_dim % 4 == 0 && row_stride % 4 == 0 && (uintptr_t)qkv % (4 * elem) == 0 &&
+                        (uintptr_t)k_cache % (4 * elem) == 0;
+  if (by_fours) {
+    const int rt = dtype == FMS_F32 ? 32 : 64;
+    FMS_REQUIRE(nheads + 2 * kvheads <= 65535, "rope_kv_write: too many heads");
+    dim3 grid(ceil_div(n_tokens, rt), nheads + 2 * kvheads);
+    const size_t lds = (size_t)rt * (head_dim + 4) * elem;
+    if (dtype == FMS_F32)
+      rope_kv_tile_kernel<float><<<grid, threads, lds, stream>>>(
+          (float*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
+          (float*)k_cache, (float*)v_cache, nheads, kvheads, head_dim, n_tokens);
+    else
+      rope_kv_tile_kernel<bf16><<<grid, threads, lds, stream>>>(
+          (bf16*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
+          (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim, n_tokens);
+  } else if (dtype == FMS_F32)
     rope_kv_write_kernel<float><<<n_tokens, threads, 0, stream>>>(
         (float*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
         (float*)k_cache, (float*)v_cache, nheads, kvheads, head_dim);
-  else if (dtype == FMS_BF16)
+  else
     rope_kv_write_kernel<bf16><<<n_tokens, threads, 0, stream>>>(
         (bf16*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
         (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim);
-  else
-    FMS_REQUIRE(false, "rope_kv_write: unknown dtype %d", dtype);
   FMS_LAUNCH_CHECK("rope_kv_write");
   return 0;
 }

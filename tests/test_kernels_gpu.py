@@ -142,7 +142,7 @@ def fill_cache(table, ks, vs, n_pages, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,K,D,rot", [(4, 2, 16, 16), (3, 1, 24, 24), (2, 2, 32, 16)])
+@pytest.mark.parametrize("H,K,D,rot", [(4, 2, 16, 16), (3, 1, 24, 24), (2, 2, 32, 16), (2, 1, 6, 6), (8, 2, 128, 128), (3, 3, 256, 64)])
 def test_rope_kv_write(ops, dtype, H, K, D, rot):
     torch.manual_seed(4)
     starts, lens = [0, 70, 5], [9, 3, 130]
