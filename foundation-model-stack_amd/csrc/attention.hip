@@ -905,27 +905,45 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   }
 }
 
-// one block per (head, token): combine the partial results of the splits
+// one block per (head, token): combine the partial results of the splits.  The loads of four splits are
+// issued together (a loop that loads, waits and combines split by split pays the memory's latency per split).
 __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                          bf16* __restrict__ out, long out_stride, const int* __restrict__ positions,
                                          const int* __restrict__ seq_of_token, int nheads, int head_dim, int n_splits,
                                          int window) {
   const int h = blockIdx.x;
   const int t = blockIdx.y;
-  if (seq_of_token[t] < 0) return;  // the decode kernel wrote zeros
-  const int pos = positions[t];
+  if (uniform_load(seq_of_token + t) < 0) return;  // the decode kernel wrote zeros
+  const int pos = uniform_load(positions + t);
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   int page_lo, page_hi;
   const int active = split_pages(lo, pos, n_splits, 0, &page_lo, &page_hi);
   const size_t base = ((size_t)t * nheads + h) * n_splits;
-  float m = -1e30f;
-  for (int s = 0; s < active; ++s) m = fmaxf(m, part_ml[(base + s) * 2]);
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float o = 0.f, l = 0.f;
-    for (int s = 0; s < active; ++s) {
-      const float f = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m);  // maxima are base-2 logarithms
-      o += f * part_o[(base + s) * head_dim + d];
-      l += f * part_ml[(base + s) * 2 + 1];
+    float m = -1e30f, o = 0.f, l = 0.f;  // running maximum (a base-2 logarithm), sum of values, sum of weights
+    for (int s0 = 0; s0 < active; s0 += 4) {
+      float ms[4], ls[4], os[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int s = s0 + i < active ? s0 + i : active - 1;  // past the end: the last split again, given no weight
+        ms[i] = part_ml[(base + s) * 2];
+        ls[i] = part_ml[(base + s) * 2 + 1];
+        os[i] = part_o[(base + s) * head_dim + d];
+      }
+      float m_new = m;
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (s0 + i < active) m_new = fmaxf(m_new, ms[i]);
+      const float keep = __builtin_amdgcn_exp2f(m - m_new);
+      o *= keep;
+      l *= keep;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float f = s0 + i < active ? __builtin_amdgcn_exp2f(ms[i] - m_new) : 0.f;
+        o += f * os[i];
+        l += f * ls[i];
+      }
+      m = m_new;
     }
     out[(size_t)t * out_stride + (size_t)h * head_dim + d] = (bf16)(l > 0.f ? o / l : 0.f);
   }
