@@ -82,6 +82,20 @@ __global__ void __launch_bounds__(GEN_THREADS)
 
 #define LOG2E 1.4426950408889634f
 
+// Maxima as single instructions.  fmaxf() first passes each operand through a max with itself (it must quiet a
+// signalling NaN), which tripled the instructions of the score maxima; the scores here come out of the matrix unit
+// and are never signalling NaNs.
+__device__ __forceinline__ float max2f(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+__device__ __forceinline__ float max3f(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 // ==========================================================================
 // MFMA core.  One wave owns 16*QT query columns and walks over pages of keys.
 // ==========================================================================
@@ -149,23 +163,19 @@ __device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&s
   for (int qt = 0; qt < QT; ++qt) {
     // maxima of the raw scores, scaled once (the scale is positive); every probability is then one fused
     // multiply-add and one exponential: exp2(s * scale2 - m)
-    float mx = -INFINITY;
-    if (full) {
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
-    } else {
+    if (!full) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int ja = key0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
         sa[qt][i] = (ja <= qpos[qt] && ja >= qlo[qt]) ? sa[qt][i] : -INFINITY;
         sb[qt][i] = (jb <= qpos[qt] && jb >= qlo[qt]) ? sb[qt][i] : -INFINITY;
-        mx = fmaxf(mx, fmaxf(sa[qt][i], sb[qt][i]));
       }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(st.m[qt], mx * scale2);
+    float mx = max3f(max3f(sa[qt][0], sa[qt][1], sa[qt][2]), max3f(sa[qt][3], sb[qt][0], sb[qt][1]), max2f(sb[qt][2], sb[qt][3]));
+    mx = max2f(mx, __shfl_xor(mx, 16, WAVE));
+    mx = max2f(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = max2f(st.m[qt], mx * scale2);
     const float alpha = __builtin_amdgcn_exp2f(st.m[qt] - m_new);
     st.m[qt] = m_new;
     float psum = 0.f;
@@ -552,23 +562,19 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
         sb = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[hf][1][c], qreg[c], sb, 0, 0, 0);
       }
     }
-    float mx = -INFINITY;
-    if (k0 + 31 <= qpos && k0 >= qlo) {  // uniform: all 32 keys are visible
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
-    } else {
+    if (!(k0 + 31 <= qpos && k0 >= qlo)) {  // uniform: not all 32 keys are visible
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int ja = k0 + g * 8 + i;  // the accumulator's rows 4 g + i hold these keys
         const int jb = ja + 4;
         sa[i] = (ja <= qpos && ja >= qlo) ? sa[i] : -INFINITY;
         sb[i] = (jb <= qpos && jb >= qlo) ? sb[i] : -INFINITY;
-        mx = fmaxf(mx, fmaxf(sa[i], sb[i]));
       }
     }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-    const float m_new = fmaxf(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
+    float mx = max3f(max3f(sa[0], sa[1], sa[2]), max3f(sa[3], sb[0], sb[1]), max2f(sb[2], sb[3]));
+    mx = max2f(mx, __shfl_xor(mx, 16, WAVE));
+    mx = max2f(mx, __shfl_xor(mx, 32, WAVE));
+    const float m_new = max2f(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
     const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
     st.m[0] = m_new;
     float pa[4], pb[4], psum = 0.f;
@@ -688,13 +694,7 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
     }
   }
 
-  float mx = -INFINITY;
-  if (key0 + PAGE_TOKENS - 1 <= qpos && key0 >= qlo) {  // uniform: all 64 keys are visible
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) mx = fmaxf(mx, fmaxf(sa[hf][i], sb[hf][i]));
-  } else {
+  if (!(key0 + PAGE_TOKENS - 1 <= qpos && key0 >= qlo)) {  // uniform: not all 64 keys are visible
 #pragma unroll
     for (int hf = 0; hf < 2; ++hf)
 #pragma unroll
@@ -703,12 +703,15 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
         const int jb = ja + 4;
         sa[hf][i] = (ja <= qpos && ja >= qlo) ? sa[hf][i] : -INFINITY;
         sb[hf][i] = (jb <= qpos && jb >= qlo) ? sb[hf][i] : -INFINITY;
-        mx = fmaxf(mx, fmaxf(sa[hf][i], sb[hf][i]));
       }
   }
-  mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-  const float m_new = fmaxf(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
+  float mx = -INFINITY;
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf)
+    mx = max3f(max3f(mx, sa[hf][0], sa[hf][1]), max3f(sa[hf][2], sa[hf][3], sb[hf][0]), max3f(sb[hf][1], sb[hf][2], sb[hf][3]));
+  mx = max2f(mx, __shfl_xor(mx, 16, WAVE));
+  mx = max2f(mx, __shfl_xor(mx, 32, WAVE));
+  const float m_new = max2f(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
   const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
   st.m[0] = m_new;
   bf16x8 pmat[2];
