@@ -90,6 +90,19 @@ __device__ __forceinline__ float max2f(float a, float b) {
   asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
   return r;
 }
+// The maximum over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (a score column's four lane groups), in all four:
+// two swaps of lane halves and rows between a register and its copy, in the vector unit (a shuffle through
+// LDS takes a round trip to LDS for each of the two steps, in the middle of the softmax's chain).
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+  const unsigned u = __float_as_uint(x);
+  const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // [lo, lo] and [hi, hi]
+  float m;
+  asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(__uint_as_float(halves[0])), "v"(__uint_as_float(halves[1])));
+  const unsigned um = __float_as_uint(m);
+  const auto rows = __builtin_amdgcn_permlane16_swap(um, um, false, false);  // rows [0, 0, 2, 2] and [1, 1, 3, 3]
+  asm("v_max_f32 %0, %1, %2" : "=v"(m) : "v"(__uint_as_float(rows[0])), "v"(__uint_as_float(rows[1])));
+  return m;
+}
 __device__ __forceinline__ float max3f(float a, float b, float c) {
   float r;
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
@@ -173,8 +186,7 @@ __device__ __forceinline__ void step_softmax(WaveState<MAXDT, QT>& st, f32x4 (&s
       }
     }
     float mx = max3f(max3f(sa[qt][0], sa[qt][1], sa[qt][2]), max3f(sa[qt][3], sb[qt][0], sb[qt][1]), max2f(sb[qt][2], sb[qt][3]));
-    mx = max2f(mx, __shfl_xor(mx, 16, WAVE));
-    mx = max2f(mx, __shfl_xor(mx, 32, WAVE));
+    mx = max_over_lane_groups(mx);
     const float m_new = max2f(st.m[qt], mx * scale2);
     const float alpha = __builtin_amdgcn_exp2f(st.m[qt] - m_new);
     st.m[qt] = m_new;
@@ -386,9 +398,11 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
   constexpr int K_ELEMS = PAGE_TOKENS * KS, V_ELEMS = MAXDT * 16 * VS;
   // at the end the same memory carries one wave's state to its partner: UNITS waves x 64 lanes x (MAXDT * 4 + 2) floats
   constexpr int MERGE_BYTES = UNITS * WAVE * (MAXDT * 4 + 2) * 4;
-  constexpr int STAGE_BYTES = (K_ELEMS + V_ELEMS) * 2 > MERGE_BYTES ? (K_ELEMS + V_ELEMS) * 2 : MERGE_BYTES;
+  // two pages: one is multiplied while the next one is written
+  constexpr int PAGE_ELEMS = K_ELEMS + V_ELEMS;
+  constexpr int STAGE_BYTES = 2 * PAGE_ELEMS * 2 > MERGE_BYTES ? 2 * PAGE_ELEMS * 2 : MERGE_BYTES;
   __shared__ __attribute__((aligned(16))) unsigned char stage[STAGE_BYTES];
-  bf16* const ks = reinterpret_cast<bf16*>(stage);
+  bf16* const ks = reinterpret_cast<bf16*>(stage);  // page b: keys at ks + b * PAGE_ELEMS, values at vs + b * PAGE_ELEMS
   bf16* const vs = ks + K_ELEMS;
 
   // Blocks of a causal step differ in length, and the longest sets the time of the whole kernel: they go
@@ -459,13 +473,13 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
       vb[j] = load_bf16x8(vp + at);
     }
   };
-  auto stash = [&](const bf16x8 (&kb)[CH], const bf16x8 (&vb)[CH]) {
+  auto stash = [&](int which, const bf16x8 (&kb)[CH], const bf16x8 (&vb)[CH]) {
 #pragma unroll
     for (int j = 0; j < CH; ++j) {
       const int id = threadIdx.x + j * THREADS;
       if (id < k_chunks) {
-        *reinterpret_cast<bf16x8*>(ks + (id / k_cols) * KS + (id % k_cols) * 8) = kb[j];
-        *reinterpret_cast<bf16x8*>(vs + (id / 8) * VS + (id % 8) * 8) = vb[j];
+        *reinterpret_cast<bf16x8*>(ks + which * PAGE_ELEMS + (id / k_cols) * KS + (id % k_cols) * 8) = kb[j];
+        *reinterpret_cast<bf16x8*>(vs + which * PAGE_ELEMS + (id / 8) * VS + (id % 8) * 8) = vb[j];
       }
     }
   };
@@ -474,23 +488,30 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
   wave_state_init(st);
   // (a fetch past the last page reads the last page again: cheaper than a branch around loads, behind which
   // the compiler loses count of the loads in flight and waits for all of them)
+  // kbuf[i % PF], vbuf[i % PF]: page page_first + i on its way from memory.  The first page goes to LDS before
+  // the loop; in the loop a page is multiplied while the next one is written to the other half of LDS and the
+  // one PF further on is asked for: one barrier a page.
+  fetch(page_first, kbuf[0], vbuf[0]);
+  stash(0, kbuf[0], vbuf[0]);
 #pragma unroll
-  for (int d = 0; d < PF; ++d) fetch(page_first + d <= page_last ? page_first + d : page_last, kbuf[d], vbuf[d]);
+  for (int d = 0; d < PF; ++d) fetch(page_first + 1 + d <= page_last ? page_first + 1 + d : page_last, kbuf[(1 + d) % PF], vbuf[(1 + d) % PF]);
+  block_sync_lds();  // not __syncthreads(): the pages under way must not be waited for
   for (int p0 = page_first; p0 <= page_last; p0 += PF) {
 #pragma unroll
     for (int d = 0; d < PF; ++d) {
-      const int pi = p0 + d;
-      if (pi > page_last) break;  // uniform
-      stash(kbuf[d], vbuf[d]);
-      block_sync_lds();  // not __syncthreads(): the pages under way must not be waited for
-      fetch(pi + PF <= page_last ? pi + PF : page_last, kbuf[d], vbuf[d]);
+      const int pi = p0 + d;  // past the last page (the loop runs in steps of PF pages): nothing but the barrier
+      const int cur = d & 1;  // PF is even: the page's half of LDS
+      if (pi + 1 <= page_last) stash(cur ^ 1, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      fetch(pi + 1 + PF <= page_last ? pi + 1 + PF : page_last, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
       const int key0 = pi * PAGE_TOKENS + khalf * 32;
-      if (has_work && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
-        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + khalf * 32 * KS, KS, vs + khalf * 32, VS, head_dim,
-                             scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
-      block_sync_lds();  // the page is overwritten next
+      if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
+        half_step<MAXDT, QT>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
+                             vs + cur * PAGE_ELEMS + khalf * 32, VS, head_dim, scale * LOG2E,
+                             key0 + 31 <= full_hi && key0 >= full_lo);
+      block_sync_lds();  // the page just multiplied is overwritten after the next one
     }
   }
+  __syncthreads();  // the loads still under way, before the memory changes its use
 
   // ---- the two waves of a unit meet: the second hands its state over, one run of 16 columns at a time ----
   const int ndt = head_dim / 16;
@@ -572,8 +593,7 @@ __device__ __forceinline__ void decode_math(WaveState<MAXDT, 1>& st, const bf16x
       }
     }
     float mx = max3f(max3f(sa[0], sa[1], sa[2]), max3f(sa[3], sb[0], sb[1]), max2f(sb[2], sb[3]));
-    mx = max2f(mx, __shfl_xor(mx, 16, WAVE));
-    mx = max2f(mx, __shfl_xor(mx, 32, WAVE));
+    mx = max_over_lane_groups(mx);
     const float m_new = max2f(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
     const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
     st.m[0] = m_new;
@@ -709,8 +729,7 @@ __device__ __forceinline__ void staged_page_step(WaveState<8, 1>& st, const bf16
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf)
     mx = max3f(max3f(mx, sa[hf][0], sa[hf][1]), max3f(sa[hf][2], sa[hf][3], sb[hf][0]), max3f(sb[hf][1], sb[hf][2], sb[hf][3]));
-  mx = max2f(mx, __shfl_xor(mx, 16, WAVE));
-  mx = max2f(mx, __shfl_xor(mx, 32, WAVE));
+  mx = max_over_lane_groups(mx);
   const float m_new = max2f(st.m[0], mx * scale2);  // the scale is positive: scaled once, after the maximum
   const float alpha = __builtin_amdgcn_exp2f(st.m[0] - m_new);
   st.m[0] = m_new;
