@@ -3,8 +3,11 @@
 //
 //   * attn_generic_kernel: any element type (float32 here), any even head
 //     size up to 256, plain FMA arithmetic.  It is the true 32-bit path.
-//   * attn_prefill_bf16_kernel / attn_decode_bf16_kernel (+ merge): bfloat16
-//     storage, float32 softmax and accumulation, MFMA 16x16x32.
+//   * attn_prefill_lds_kernel (pages through LDS, shared by the heads of a kv
+//     group), attn_prefill_bf16_kernel (straight from global memory: head
+//     sizes and head groups the first does not take) and
+//     attn_decode_bf16_kernel (+ merge): bfloat16 storage, float32 softmax and
+//     accumulation, MFMA 16x16x32.
 //
 // The MFMA kernels compute S^T = K Q^T (rows: keys, columns: queries) so that
 // the probabilities come out of the accumulator already in the operand layout
@@ -371,12 +374,13 @@ __global__ void __launch_bounds__(WAVES* WAVE)
 }
 
 // ==========================================================================
-// prefill through LDS.  A block stages one page of keys and values at a time
-// in LDS.  It has four units: `hb` query heads of one kv group (they share the
-// page) times 4/hb runs of 16*QT consecutive query tokens; a unit is two waves
-// that take one half of every page each and meet at the end, which halves the
-// chain of dependent steps of the longest block of a causal step.  The next
-// page is fetched into registers while the current one is multiplied.
+// prefill through LDS.  A block stages the pages of keys and values in LDS,
+// two at a time: one is multiplied while the next is written.  It has four
+// units: `hb` query heads of one kv group (they share the page) times 4/hb runs
+// of 16*QT consecutive query tokens; a unit is two waves that take one half of
+// every page each and meet at the end, which halves the chain of dependent
+// steps of the longest block of a causal step.  Pages are fetched into
+// registers two ahead of the one that is multiplied.
 // ==========================================================================
 #define LDS_PAD 8  // elements: rows 16 bytes apart from a multiple of the bank count
 
@@ -556,11 +560,12 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
 
 // ==========================================================================
 // decode: one query token per sequence.  Grid (split, kv head x head tile,
-// token); a block is ONE wave whose 16 columns are query heads that share the
-// kv head.  A split covers `pages_per_split` pages.  Small blocks in large
-// numbers keep the whole cache of a small batch in flight at once; the loads
-// of a page (keys and values) are issued together before any arithmetic.
-// Splits of one token meet in attn_decode_merge_kernel.
+// token); the 16 columns of a wave's tiles are query heads that share the kv
+// head.  Every sequence deals its own pages out over the splits; the waves of
+// a block (up to 8) take the pages of its split in turn and meet in LDS; the
+// splits of a token meet in attn_decode_merge_kernel.  For a small batch many
+// small blocks keep the whole cache in flight at once; for a large one a block
+// takes a whole sequence, and the long sequences go first.
 // ==========================================================================
 // The arithmetic of HALVES halves of 32 keys starting at key0, for operands that are already in registers:
 // kreg[hf][tile][c] the keys of the two score tiles (rows dealt as key_a below says), vreg[hf][dt] the values.
