@@ -351,6 +351,22 @@ def test_block_table_rows_follow_the_step_order():
     assert set(table.flatten().tolist()) - {-1} == set(cache.groups[0].pages[a] + cache.groups[0].pages[b])
 
 
+def test_a_decode_batch_lists_its_rows_longest_context_first():
+    from fms_amd.engine.batch import build_batch
+
+    cache = make_cache(max_tokens=64 * 12, max_slots=5)
+    slots = [cache.alloc_slot() for _ in range(4)]
+    for slot, n in zip(slots, (5, 130, 64, 70)):
+        cache.extend(slot, n)
+    starts = [cache.extend(slot, 1) for slot in slots]
+    batch = build_batch(cache, slots, [[1], [2], [3], [4]], starts, [[0]] * 4, "cpu")
+    assert batch.is_decode and batch.rows_by_length.tolist() == [1, 3, 2, 0]
+    # a step that brings a prompt has no such order
+    other = cache.alloc_slot()
+    batch = build_batch(cache, [other], [[1, 2, 3]], [cache.extend(other, 3)], [[2]], "cpu")
+    assert not batch.is_decode and batch.rows_by_length is None
+
+
 # --------------------------------------------------------------------------
 # generation loop
 # --------------------------------------------------------------------------
