@@ -12,8 +12,6 @@ from __future__ import annotations
 import re
 from typing import List, Tuple
 
-import torch
-
 from ..config import LLaMAConfig
 from ..config.llama import HF_ARCHITECTURES
 from ..parts import LayerSpec, ModelSpec, PartSpec

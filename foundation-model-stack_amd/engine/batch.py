@@ -9,7 +9,7 @@ from typing import Dict, List, Optional, Sequence
 
 import torch
 
-from ..cache import PAGE_TOKENS, SequenceCache
+from ..cache import SequenceCache
 
 
 @dataclasses.dataclass

@@ -17,11 +17,11 @@ from __future__ import annotations
 
 import gc
 
-from typing import Dict, List, Optional, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import torch
 
-from ..cache import PAGE_TOKENS, pages_for
+from ..cache import pages_for
 from ..kernels import ops
 from .batch import StepBatch
 

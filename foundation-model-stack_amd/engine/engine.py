@@ -16,7 +16,6 @@ import torch
 import os
 
 from ..cache import CacheFull, pages_for
-from ..kernels import ops
 from ..sampling import SamplingParams, choose
 from .batch import StepBatch, build_batch
 from .decode_graph import CONTEXT_HEADROOM, DecodeGraph, context_bucket, row_bucket

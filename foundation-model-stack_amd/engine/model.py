@@ -3,7 +3,7 @@ order of the schedule, final norm, head.  It knows no architecture by name."""
 
 from __future__ import annotations
 
-from typing import Dict, List, Optional, Tuple
+from typing import List, Optional, Tuple
 
 import torch
 

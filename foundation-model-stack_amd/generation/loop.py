@@ -13,7 +13,7 @@ the model's last position; its slot goes back at once and the batch shrinks.
 from __future__ import annotations
 
 import time
-from typing import Callable, Iterable, List, Optional, Sequence, Set, Union
+from typing import Callable, Iterable, List, Optional, Sequence, Set
 
 import torch
 

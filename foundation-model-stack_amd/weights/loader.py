@@ -13,11 +13,10 @@ from __future__ import annotations
 
 import hashlib
 import re
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, List, Optional
 
 import torch
 
-from ..parts import Part
 from .adapters import get_adapter
 from .checkpoint import Checkpoint
 

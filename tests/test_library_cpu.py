@@ -15,7 +15,7 @@ from fms_amd.config import LLaMAConfig
 from fms_amd.engine.model import DecoderModel
 from fms_amd.architectures.llama import detect_source, llama_spec
 from fms_amd.generation import generate_requests, pad_input_ids, plan_batches, trim_prefix, truncate_after_eos
-from fms_amd.parts import ModelSpec, ScheduleEntry
+from fms_amd.parts import ScheduleEntry
 from fms_amd.weights import Checkpoint, WeightsError, get_adapter, kept_dtype, load_checkpoint, write_safetensors
 
 import plain_llama as P
