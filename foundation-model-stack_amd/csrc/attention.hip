@@ -66,7 +66,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
     const float psum = block_sum(p, scratch);  // has the barriers that publish ps
     l_run = l_run * alpha + psum;
     m_run = m_new;
-    if (threadIdx.x < head_dim) {
+    if ((int)threadIdx.x < head_dim) {
       const int d = threadIdx.x;
       float a = acc * alpha;
       const int n = pos - base + 1 < GEN_THREADS ? pos - base + 1 : GEN_THREADS;
@@ -80,7 +80,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
     }
     __syncthreads();  // ps is overwritten by the next chunk
   }
-  if (threadIdx.x < head_dim) o[threadIdx.x] = from_f32<T>(l_run > 0.f ? acc / l_run : 0.f);
+  if ((int)threadIdx.x < head_dim) o[threadIdx.x] = from_f32<T>(l_run > 0.f ? acc / l_run : 0.f);
 }
 
 #define LOG2E 1.4426950408889634f
