@@ -7,6 +7,7 @@ from __future__ import annotations
 import dataclasses
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache import SequenceCache
@@ -51,20 +52,20 @@ def build_batch(
     B = len(slots)
     q_lens = [len(t) for t in tokens]
     T = sum(q_lens)
-    flat_ids: List[int] = []
-    positions: List[int] = []
-    seq_of_token: List[int] = []
-    seq_starts = [0]
+    # arrays, not Python loops over tokens: a prompt of thousands of tokens is prepared while the GPU waits
+    lens = np.asarray(q_lens, dtype=np.int64)
+    first = np.asarray(list(starts), dtype=np.int64)
+    offsets = np.concatenate([[0], np.cumsum(lens)])
+    seq_of_token = np.repeat(np.arange(B, dtype=np.int64), lens)
+    flat_ids = np.concatenate([np.asarray(t, dtype=np.int64) for t in tokens]) if B else np.zeros(0, dtype=np.int64)
+    positions = np.arange(T, dtype=np.int64) - offsets[:-1][seq_of_token] + first[seq_of_token]
+    seq_starts = offsets
     rows: List[int] = []
     sizes = sorted(set(int(s) for s in qblock_sizes if s))
     qb_start: Dict[int, List[int]] = {s: [] for s in sizes}
     qb_len: Dict[int, List[int]] = {s: [] for s in sizes}
     for b in range(B):
-        base = seq_starts[-1]
-        flat_ids.extend(int(x) for x in tokens[b])
-        positions.extend(range(starts[b], starts[b] + q_lens[b]))
-        seq_of_token.extend([b] * q_lens[b])
-        seq_starts.append(base + q_lens[b])
+        base = int(offsets[b])
         for w in want[b]:
             if not 0 <= w < q_lens[b]:
                 raise IndexError(f"wanted place {w} is outside the {q_lens[b]} tokens of sequence {b}")
@@ -77,7 +78,7 @@ def build_batch(
 
     # one host buffer, one copy
     is_decode = all(n == 1 for n in q_lens)
-    by_length = sorted(range(T), key=lambda t: -positions[t]) if is_decode else []
+    by_length = np.argsort(-positions, kind="stable") if is_decode else []
     parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows, by_length]
     for size in sizes:
         parts += [qb_start[size], qb_len[size]]
@@ -89,7 +90,7 @@ def build_batch(
     spans = []
     for p, n in zip(parts, lengths):
         if n:
-            host[off : off + n] = torch.tensor(p, dtype=torch.int32)
+            host[off : off + n] = torch.from_numpy(np.asarray(p).astype(np.int32, copy=False))
         spans.append((off, n))
         off += n
     table_spans = {}
