@@ -4,8 +4,8 @@
 //   * attn_generic_kernel: any element type (float32 here), any even head
 //     size up to 256, plain FMA arithmetic.  It is the true 32-bit path.
 //   * attn_prefill_lds_kernel (pages through LDS, shared by the heads of a kv
-//     group), attn_prefill_bf16_kernel (straight from global memory: head
-//     sizes and head groups the first does not take) and
+//     group; head sizes up to 128), attn_prefill_bf16_kernel (straight from
+//     global memory; head sizes above 128) and
 //     attn_decode_bf16_kernel (+ merge): bfloat16 storage, float32 softmax and
 //     accumulation, MFMA 16x16x32.
 //
