@@ -65,12 +65,14 @@ def generate_requests(
     chooser: Optional[Callable] = None,
     on_step: Optional[Callable[[int, List[int], List[int]], None]] = None,
     step_times: Optional[List[float]] = None,
+    before_step: Optional[Callable[[int, List[int], List[List[int]]], Optional[List[List[int]]]]] = None,
 ) -> List[List[int]]:
     """New tokens of every request (a stop token is kept, nothing follows it).
 
     engine: anything with new_sequence(), end_sequence(slot), step(slots, tokens, want), and
     cache.max_tokens / cache.max_slots / cache.max_seq_len.  chooser(logits, request_indices,
-    counters) -> token ids overrides the built-in sampler (tests use it).
+    counters) -> token ids overrides the built-in sampler (tests use it).  before_step(step, requests, tokens)
+    sees the tokens each live request is about to be fed and may return others in their place (as many lists).
     """
     sampling = sampling or SamplingParams(do_sample=False)
     stops: Set[int] = set(int(s) for s in (stop_token_ids or ()))
@@ -95,8 +97,15 @@ def generate_requests(
         step_no = 0
         try:
             while alive:
+                if before_step is not None:
+                    given = before_step(step_no, list(alive), [list(feed[r]) for r in alive])
+                    if given is not None:
+                        if len(given) != len(alive) or any(len(g) == 0 for g in given):
+                            raise ValueError("before_step must return one non-empty token list per live request")
+                        for r, g in zip(alive, given):
+                            feed[r] = [int(x) for x in g]
                 t0 = time.time()
-                if fused and step_no > 0:
+                if fused and step_no > 0 and all(len(feed[r]) == 1 for r in alive):
                     # decode: the step and the choice in one call (a captured graph when the engine has one)
                     tokens = engine.decode_and_choose(
                         [slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
@@ -200,6 +209,7 @@ def generate(
     eos_token_id: Optional[int] = None,
     pad_token_id: Optional[int] = None,
     timing: str = "",
+    prepare_model_inputs_hook: Optional[Callable] = None,
     post_iteration_hook: Optional[Callable] = None,
     extra_kwargs: Optional[dict] = None,
     seed: int = 0,
@@ -211,6 +221,10 @@ def generate(
     a row that ended early is filled up with eos_token_id (or pad_token_id, or 0).
     use_cache / contiguous_cache are accepted for compatibility: the engine always caches.
     With timing "per-token" or "e2e" returns (result, times) as the reference does.
+    prepare_model_inputs_hook(i, input_ids, kwargs) -> (input_ids, kwargs) is called before step i, as in the
+    reference (fms/utils/generation.py:295-296), with the tokens about to be fed as a tensor [rows alive, n]
+    (left-padded with pad_token_id or 0 where the rows differ in length) and the extra_kwargs; the tokens it
+    returns are fed instead (the same shape; padding places are ignored).
     """
     from ..engine import Engine  # late import: engine imports the kernels
 
@@ -226,6 +240,17 @@ def generate(
     engine = model if isinstance(model, Engine) else default_engine(model, prompts, max_new_tokens)
     times: List[float] = []
     start = time.time()
+    before = None
+    if prepare_model_inputs_hook is not None:
+        pad = pad_token_id if pad_token_id is not None else 0
+        state = {"kwargs": dict(extra_kwargs or {})}
+
+        def before(step, alive, tokens):
+            width = max(len(t) for t in tokens)
+            ids = torch.tensor([[pad] * (width - len(t)) + list(t) for t in tokens], dtype=ids2d.dtype)
+            ids, state["kwargs"] = prepare_model_inputs_hook(step, ids, state["kwargs"])
+            return [row[width - len(t):] for row, t in zip(ids.tolist(), tokens)]
+
     hook = None
     if post_iteration_hook is not None:
         hook = lambda step, alive, tokens: post_iteration_hook(step, alive, tokens)  # noqa: E731
@@ -238,6 +263,7 @@ def generate(
         seed=seed,
         on_step=hook,
         step_times=times if timing == "per-token" else None,
+        before_step=before,
     )
     if timing == "e2e":
         if engine.device.type == "cuda":

@@ -277,6 +277,21 @@ def test_greedy_generation_through_the_entry_point(lib, folders, name):
     for b, (p, w) in enumerate(zip(prompts, want)):
         assert out[b].tolist()[-16:] == w
         assert out[b].tolist()[20 - len(p) : 20] == p
+    # the reference's hook before every step: it sees what is about to be fed (rows padded on the left) and may
+    # change it; here it puts the second prompt in the first one's place at step 0 and leaves the rest alone
+    calls = []
+
+    def swap_first_prompt(i, input_ids, kwargs):
+        calls.append((i, tuple(input_ids.shape), kwargs.get("note")))
+        if i == 0:
+            input_ids = input_ids.clone()
+            input_ids[0, -len(prompts[0]) :] = torch.tensor(prompts[1][-len(prompts[0]) :])
+        return input_ids, kwargs
+
+    out = generate(model, torch.tensor(prompts[0]), max_new_tokens=4, do_sample=False, prepare_model_inputs_hook=swap_first_prompt,
+                   extra_kwargs={"note": "kept"})
+    assert out.tolist()[len(prompts[0]) :] == P.greedy_generate(weights, cfg, prompts[1][-len(prompts[0]) :], 4)
+    assert calls[0] == (0, (1, len(prompts[0])), "kept") and calls[1] == (1, (1, 1), "kept") and len(calls) == 4
     # a stop token ends its own request only
     stop = want[1][3]
     out = generate(model, ids, max_new_tokens=16, do_sample=False, extra_kwargs=extra, eos_token_id=stop)

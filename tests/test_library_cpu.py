@@ -427,6 +427,25 @@ def test_loop_unequal_prompts_stops_and_limits():
     assert generate_requests(engine, [[1]], max_new_tokens=0, chooser=argmax_chooser) == [[]]
 
 
+def test_loop_lets_a_hook_change_what_is_fed():
+    """before_step sees the tokens about to be fed and may replace them (the reference's
+    prepare_model_inputs_hook, fms/utils/generation.py:295-296, reaches the loop through it)."""
+    engine = FakeEngine()
+    seen = []
+
+    def hook(step, requests, tokens):
+        seen.append((step, list(requests), [list(t) for t in tokens]))
+        if step == 2:
+            return [[40] for _ in tokens]  # from here the mock counts on from 40
+        return None
+
+    out = generate_requests(engine, [[10, 11], [20]], max_new_tokens=4, chooser=argmax_chooser, before_step=hook)
+    assert out == [[12, 13, 41, 42], [21, 22, 41, 42]]
+    assert seen[0] == (0, [0, 1], [[10, 11], [20]]) and seen[1] == (1, [0, 1], [[12], [21]]) and seen[2][2] == [[13], [22]]
+    with pytest.raises(ValueError):
+        generate_requests(FakeEngine(), [[1]], max_new_tokens=2, chooser=argmax_chooser, before_step=lambda s, r, t: [])
+
+
 def test_loop_runs_as_many_batches_as_the_requests_need():
     engine = FakeEngine(max_tokens=64 * 2, max_slots=2)
     prompts = [[i] for i in range(7)]
