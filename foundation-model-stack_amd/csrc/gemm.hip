@@ -208,10 +208,11 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE) __attribute__((amdgpu_waves_pe
   const int wave = threadIdx.x / WAVE;
   const int lane = threadIdx.x & (WAVE - 1);
   const int r = lane & 15, g = lane >> 4;
-  // A block owns rows_per_block rows of W (a multiple of 8, at most 16 * NTB; its last tile may be partly
-  // empty): 24 rows make 256 equal blocks of 6144 rows where 16 would make 384.  Gated: 16 and 16.
-  const int n0 = blockIdx.x * (GATED ? 16 : rows_per_block);
-  const int n_end = GATED ? N : (n0 + rows_per_block < N ? n0 + rows_per_block : N);
+  // A block owns rows_per_block rows of W (at most 16 * NTB; its last tile may be partly
+  // empty): 24 rows make 256 equal blocks of 6144 rows where 16 would make 384.  Gated: that many gate rows in the
+  // first tile and their up rows in the second.
+  const int n0 = blockIdx.x * rows_per_block;
+  const int n_end = n0 + rows_per_block < N ? n0 + rows_per_block : N;
 
   if (EPI == EPI_ROPE && threadIdx.x < MT * 16) {
     // index data of the rows, fetched while the weights stream
@@ -311,7 +312,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE) __attribute__((amdgpu_waves_pe
 #pragma unroll
       for (int t = 0; t < NTB; ++t) {
         const int nbase = n0 + (t == 0 ? 0 : (GATED ? tile2_offset : 16 * t));
-        const int limit = GATED ? (t == 0 ? N : tile2_offset + N) : n_end;
+        const int limit = GATED && t == 1 ? tile2_offset + n_end : n_end;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           // a row past the block's last is read from the block's first (its sums are never stored), a piece
@@ -487,7 +488,7 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
                           int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int rows_per_block,
                           hipStream_t stream, RowScale scale, RopeEpilogue rope = RopeEpilogue{},
                           ResidEpilogue res = ResidEpilogue{}) {
-  const int blocks = ceil_div(N, EPI == EPI_GATED ? 16 : rows_per_block);
+  const int blocks = ceil_div(N, rows_per_block);
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
   constexpr int SK_WAVES = 8;
   constexpr int UNR = (NTB + MT) <= 2 ? 2 : 1;
@@ -509,17 +510,33 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
 #undef FMS_SK
 }
 
-// Rows of W per block (16, 24 or 32) for a product of N rows: the choice that costs the fewest rounds of
-// blocks over the compute units, a round costing as much as its blocks have rows.  Large products take 32
-// (the activations are then read once per two tiles).
+// Rows of W per block.  The blocks are dealt over the compute units (one or two at a time on each, sharing its
+// path to memory), and what a unit has to pull decides the time: its blocks' weight rows and, per block, the
+// rows of x (read four rows an instruction).  The choice with the least of
+//   blocks per unit (a whole number) x (rows of W + rows of x per block)
+// wins: 6144 rows in blocks of 24 are one block a unit where blocks of 16 are one and a half; the gated product
+// of 14336 columns in blocks of 14 gate rows and 14 up rows is four blocks a unit of 28 rows where blocks of 16
+// and 16 are three and a half - that is, four for some - of 32.
 #define SK_COMPUTE_UNITS 256
-static int skinny_rows_per_block(int N) {
-  if (N >= 16384) return 32;
-  int best = 16;
+static int skinny_x_rows(int M) { return ceil_div(M < 16 ? M : 16, 4) * 4; }
+
+static int skinny_rows_per_block(int N, int M) {
+  int best = 0;
   long best_cost = 0;
-  for (int rows = 16; rows <= 32; rows += 8) {
-    const long cost = (long)ceil_div(ceil_div(N, rows), SK_COMPUTE_UNITS) * rows;
-    if (rows == 16 || cost < best_cost) best = rows, best_cost = cost;
+  for (int rows = 12; rows <= 32; rows += 2) {
+    const long cost = (long)ceil_div(ceil_div(N, rows), SK_COMPUTE_UNITS) * (rows + skinny_x_rows(M));
+    if (best == 0 || cost <= best_cost) best = rows, best_cost = cost;  // a tie goes to the larger blocks
+  }
+  return best;
+}
+
+// gate rows (and as many up rows) per block of the gated product
+static int skinny_gated_rows_per_block(int hidden, int M) {
+  int best = 0;
+  long best_cost = 0;
+  for (int rows = 12; rows <= 16; ++rows) {
+    const long cost = (long)ceil_div(ceil_div(hidden, rows), SK_COMPUTE_UNITS) * (2 * rows + skinny_x_rows(M));
+    if (best == 0 || cost <= best_cost) best = rows, best_cost = cost;
   }
   return best;
 }
@@ -548,7 +565,7 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   if (M > 16)
     return wide_product(EPI_PLAIN, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, scale, RopeEpilogue{},
                         ResidEpilogue{}, workspace, workspace_bytes, stream);
-  const int rows = skinny_rows_per_block(N);
+  const int rows = skinny_rows_per_block(N, M);
 #define FMS_LS(NTB, MT) \
   launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, rows, stream, scale)
   if (rows > 16)
@@ -579,8 +596,8 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
     return wide_product(EPI_GATED, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, scale,
                         RopeEpilogue{}, ResidEpilogue{}, workspace, workspace_bytes, stream);
 #define FMS_LG(MT) \
-  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, 16, \
-                                  stream, scale)
+  launch_skinny<2, MT, EPI_GATED>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act,     \
+                                  skinny_gated_rows_per_block(hidden, M), stream, scale)
   FMS_LG(1);
 #undef FMS_LG
   FMS_LAUNCH_CHECK("gemm_skinny_gated_bf16");
@@ -616,7 +633,7 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   if (M > 16)
     return wide_product(EPI_ROPE, x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, scale, rope,
                         ResidEpilogue{}, workspace, workspace_bytes, stream);
-  const int rows = skinny_rows_per_block(N);
+  const int rows = skinny_rows_per_block(N, M);
 #define FMS_LR(NTB, MT) \
   launch_skinny<NTB, MT, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
   if (rows > 16)
@@ -638,7 +655,7 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
 // normed stream.  M <= 64.
 extern "C" int fmsamd_gemm_skinny_residual_partials(int M, int N) {
   if (M > 16) return ceil_div(N, 16);
-  const int rows = skinny_rows_per_block(N);
+  const int rows = skinny_rows_per_block(N, M);
   return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
 }
 
@@ -663,7 +680,7 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
   FMS_REQUIRE(resid != nullptr && scaled != nullptr && partials != nullptr, "gemm_skinny_residual_bf16: null buffer");
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
-  const int rows = skinny_rows_per_block(N);
+  const int rows = skinny_rows_per_block(N, M);
   const int tiles = fmsamd_gemm_skinny_residual_partials(M, N);
   FMS_REQUIRE(partial_count >= tiles, "gemm_skinny_residual_bf16: room for %d partial sums per row, %d needed",
               partial_count, tiles);
