@@ -27,6 +27,7 @@ struct WideOut {
   const void* bias;
   int bias_f32;
   int N, tile2_offset, act;
+  int gate_rows;  // WD_GATED: gate rows (and up rows) a block owns, a multiple of 4, at most 64
   int vec;  // rows of the destination start 16-byte aligned: four elements at a time
   RowScale scale;
 };
@@ -62,9 +63,10 @@ __global__ void __launch_bounds__(512)
   // the wave's 16 weight rows start at n0; rows from n_end on are not the wave's to read
   int n0 = blockIdx.x * WD_ROWS + wave * 16, n_end = rows;
   if (MODE == WD_GATED) {
-    const int first = blockIdx.x * (WD_ROWS / 2) + (wave & 3) * 16;
+    const int first = blockIdx.x * o.gate_rows + (wave & 3) * 16;
+    const int last = (blockIdx.x + 1) * o.gate_rows < o.N ? (blockIdx.x + 1) * o.gate_rows : o.N;  // the block's end
     n0 = wave < 4 ? first : o.tile2_offset + first;
-    n_end = wave < 4 ? o.N : o.tile2_offset + o.N;
+    n_end = wave < 4 ? last : o.tile2_offset + last;
   }
   const int ngroups = (K + WD_GROUP - 1) / WD_GROUP;
   const int g_begin = blockIdx.y * groups_per_slice;
@@ -204,12 +206,13 @@ __global__ void __launch_bounds__(512)
   if (MODE == WD_GATED) {
     // 16 threads a row: four gate columns and their four up columns each
     const int c = 4 * (threadIdx.x & 15);
-    const int n = blockIdx.x * (WD_ROWS / 2) + c;
+    const int n = blockIdx.x * o.gate_rows + c;
+    const int n_hi = (blockIdx.x + 1) * o.gate_rows < o.N ? (blockIdx.x + 1) * o.gate_rows : o.N;
     OutT* const out = (OutT*)o.out;
 #pragma unroll
     for (int p = 0; p < (MT + 1) / 2; ++p) {
       const int m = p * 32 + (threadIdx.x >> 4);
-      if (m >= M || m >= MT * 16 || n >= o.N) continue;
+      if (m >= M || m >= MT * 16 || n >= n_hi) continue;
       const f32x4 gate = *reinterpret_cast<const f32x4*>(tile + m * WD_TILE_LD + c);
       const f32x4 up = *reinterpret_cast<const f32x4*>(tile + m * WD_TILE_LD + WD_ROWS / 2 + c);
       const float rs = row_scale[m];
@@ -217,18 +220,18 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         float v = gate[e] * rs, u = up[e] * rs;
-        if (o.bias != nullptr && n + e < o.N) {
+        if (o.bias != nullptr && n + e < n_hi) {
           v += wide_bias(o, n + e);
           u += wide_bias(o, o.tile2_offset + n + e);
         }
         res[e] = sk_activate(v, o.act) * u;
       }
-      if (o.vec && n + 3 < o.N) {
+      if (o.vec && n + 3 < n_hi) {
         store4(out + (size_t)m * o.ldo + n, res);
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          if (n + e < o.N) out[(size_t)m * o.ldo + n + e] = from_f32<OutT>(res[e]);
+          if (n + e < n_hi) out[(size_t)m * o.ldo + n + e] = from_f32<OutT>(res[e]);
       }
     }
   } else {
@@ -431,6 +434,19 @@ static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float
 #undef FMS_WK
 }
 
+// Gate rows per block of a gated product that finishes in one kernel: what a compute unit has to pull is its
+// blocks (a whole number) times a block's rows of W and of x; 14336 columns in blocks of 64 are 224 blocks for 256
+// units, in blocks of 56 one block for each.
+static int wide_gate_rows(int M, int N) {
+  int best = 0;
+  long best_cost = 0;
+  for (int rows = 32; rows <= WD_ROWS / 2; rows += 4) {
+    const long cost = (long)ceil_div(ceil_div(N, rows), WD_COMPUTE_UNITS) * (2 * rows + M);
+    if (best == 0 || cost <= best_cost) best = rows, best_cost = cost;
+  }
+  return best;
+}
+
 static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 // N: columns of the output (for the gated product the hidden size; W then has tile2_offset + N rows).
@@ -443,13 +459,14 @@ int wide_product(int epi, const void* x, long ldx, const void* w, const void* bi
   const int ngroups = ceil_div(K, WD_GROUP);
   const int per_slice = ceil_div(ngroups, slices);
   const bool itself = slices == 1 && wide_finishes_itself(epi);
-  WideOut o{out, ldo, bias, bias != nullptr && bias_dtype == FMS_F32, N, tile2_offset, act, 0, scale};
+  WideOut o{out, ldo, bias, bias != nullptr && bias_dtype == FMS_F32, N, tile2_offset, act, WD_ROWS / 2, 0, scale};
 
   if (itself) {
     const long elem = out_dtype == FMS_BF16 ? 2 : 4;
     o.vec = ((uintptr_t)out % (4 * elem)) == 0 && ldo % 4 == 0;
     if (epi == EPI_GATED) {
-      dim3 grid(ceil_div(N, WD_ROWS / 2), 1);
+      o.gate_rows = wide_gate_rows(M, N);
+      dim3 grid(ceil_div(N, o.gate_rows), 1);
       if (out_dtype == FMS_BF16)
         launch_wide<WD_GATED, bf16>(grid, x, ldx, w, nullptr, M, rows, K, per_slice, o, stream);
       else
