@@ -33,6 +33,8 @@ def main() -> int:
     ap.add_argument("--variant", default="3-8b")
     ap.add_argument("--context", type=int, default=8192)
     ap.add_argument("--prefill-tokens", type=int, default=2048)
+    ap.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
+    ap.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches")
     ap.add_argument("--skip-points", action="store_true", help="leave out decode at batch 1 and 64")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
@@ -65,13 +67,14 @@ def main() -> int:
 
     def decode(batch: int, steps: int, warmup: int):
         """(tokens/s, ms per step, bytes a step has to read) for `batch` sequences with prompts of 128..2048 tokens."""
-        lens = [rng.randint(128, 2048) for _ in range(batch)]
+        lens = [rng.randint(args.prompt_min, args.prompt_max) for _ in range(batch)]
         room = sum(-(-(n + steps + warmup + 1) // 64) * 64 for n in lens)
         engine = Engine(model, max_tokens=room, max_slots=batch)
         slots = [engine.new_sequence() for _ in range(batch)]
         tokens = None
-        for i in range(0, batch, 8):  # prompts in groups, so that activations stay small
-            group = list(range(i, min(i + 8, batch)))
+        per_group = max(1, 16384 // args.prompt_max)  # prompts in groups, so that activations stay small
+        for i in range(0, batch, per_group):
+            group = list(range(i, min(i + per_group, batch)))
             prompts = [[rng.randrange(V) for _ in range(lens[b])] for b in group]
             logits = engine.step([slots[b] for b in group], prompts, "last")
             first = choose(logits, greedy).tolist()
@@ -120,11 +123,17 @@ def main() -> int:
     achieved = step_bytes / (ms / 1000) / 1e9 if ms else 0.0
     points = {}
     if not args.skip_points and args.only is None:
-        points["decode_b1"] = round(decode(1, min(args.steps, 32), 4)[0], 1)
-        points["decode_b64"] = round(decode(64, min(args.steps, 16), 2)[0], 1)
+        for b, steps, warmup in ((1, min(args.steps, 32), 4), (64, min(args.steps, 16), 2)):
+            p_tps, p_ms, p_bytes = decode(b, steps, warmup)
+            gbs = p_bytes / (p_ms / 1000) / 1e9
+            points[f"decode_b{b}"] = round(p_tps, 1)
+            points[f"decode_b{b}_ms"] = round(p_ms, 3)
+            points[f"decode_b{b}_gb"] = round(p_bytes / 1e9, 3)
+            points[f"decode_b{b}_gbs"] = round(gbs, 1)
+            points[f"decode_b{b}_frac"] = round(gbs / HBM_GBS, 4)
 
     record = {
-        "metric": "decode tok/s at batch 8 (Llama-3-8B shape, 8192 context); prefill tok/s at 2048 tokens",
+        "metric": f"decode tok/s at batch {args.batch} (llama {args.variant} shape, {args.context} context); prefill tok/s at {args.prefill_tokens} tokens",
         "value": round(tps, 1),
         "unit": "tokens/s",
         "n_gpus": 1,
@@ -135,7 +144,7 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic: random weights N(0, 0.02), uniform random token ids, prompt lengths uniform in [128, 2048]",
+        "data": f"synthetic: random weights N(0, 0.02), uniform random token ids, prompt lengths uniform in [{args.prompt_min}, {args.prompt_max}]",
         "config": {
             "model": f"llama {args.variant} shape",
             "global_batch": args.batch,
@@ -151,8 +160,8 @@ def main() -> int:
             "vocab": V,
             "rope_theta": cfg.rope_theta,
             "norm_eps": cfg.norm_eps,
-            "prompt_len_min": 128,
-            "prompt_len_max": 2048,
+            "prompt_len_min": args.prompt_min,
+            "prompt_len_max": args.prompt_max,
             "prefill_tokens": args.prefill_tokens,
             "cache_page_tokens": 64,
         },

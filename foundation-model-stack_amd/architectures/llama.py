@@ -195,6 +195,7 @@ register_architecture(
         from_hf_dict=LLaMAConfig.from_hf_dict,
         to_hf_dict=LLaMAConfig.to_hf_dict,
         hf_tensor_layout=hf_tensor_layout,
+        detect_source=detect_source,
     )
 )
 

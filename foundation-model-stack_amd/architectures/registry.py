@@ -23,6 +23,7 @@ class Architecture:
     from_hf_dict: Callable[[dict], ModelConfig] = None  # config.json (Hugging Face keys) -> configuration
     to_hf_dict: Callable[[ModelConfig], dict] = None
     hf_tensor_layout: Callable[[ModelConfig], list] = None  # names/shapes/inits of a Hugging Face checkpoint
+    detect_source: Callable[[list], str] = None  # a checkpoint's tensor names -> the name of its source (adapter)
 
 
 _architectures: Dict[str, Architecture] = {}

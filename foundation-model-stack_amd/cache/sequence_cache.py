@@ -103,6 +103,8 @@ class SequenceCache:
 
         self._free_slots: List[int] = list(range(max_slots - 1, -1, -1))
         self._live: Dict[int, int] = {}  # slot -> length
+        self._clock = 0
+        self._stamp: Dict[int, int] = {}  # slot -> value of the clock at its last change
         if device is not None:
             for group in self.groups:
                 group.allocate_storage(dtype, device)
@@ -120,6 +122,8 @@ class SequenceCache:
         if slot in self._live:
             raise AssertionError(f"slot {slot} was free while live")
         self._live[slot] = 0
+        self._clock += 1
+        self._stamp[slot] = self._clock
         for group in self.groups:
             group.pages[slot] = []
         for tensors in self.state.values():
@@ -135,6 +139,7 @@ class SequenceCache:
                 if page >= 0:
                     group.pool.free(page)
         del self._live[slot]
+        del self._stamp[slot]
         self._free_slots.append(slot)
 
     def live_slots(self) -> List[int]:
@@ -149,28 +154,24 @@ class SequenceCache:
 
     # ---- pages -----------------------------------------------------------
     def pages_needed(self, slot: int, new_tokens: int) -> int:
-        """Pages the full-length groups would have to take for `new_tokens` more tokens (the most of any group)."""
-        new_len = self._live[slot] + new_tokens
+        """Pages that `new_tokens` more tokens of `slot` take from the pools (the most of any group), counting
+        the pages a windowed group gives back first."""
         need = 0
-        for group in self.groups:
-            need = max(need, pages_for(new_len) - len(group.pages[slot]))
+        for _, release, want in self._plan(slot, new_tokens):
+            need = max(need, want - len(release))
         return max(need, 0)
 
-    def extend(self, slot: int, new_tokens: int) -> int:
-        """Make room for `new_tokens` more tokens of `slot`; returns the position of the first of them.
-
-        Windowed groups first give back the pages that no query of this step can see.
-        Nothing changes if the room cannot be made.
-        """
+    def _plan(self, slot: int, new_tokens: int):
+        """For every group: (group, indices of the slot's pages that no query of the step can see any more,
+        pages to take).  Changes nothing."""
         if slot not in self._live:
             raise ValueError(f"slot {slot} is not live")
-        start = self._live[slot]
-        new_len = start + new_tokens
         if new_tokens < 0:
             raise ValueError("a sequence cannot shrink")
+        start = self._live[slot]
+        new_len = start + new_tokens
         if new_len > self.max_seq_len:
-            raise IndexError(f"sequence of {new_len} tokens exceeds the model's {self.max_seq_len} positions")
-        # which pages would be released, and is there room afterwards?
+            raise IndexError(f"sequence in slot {slot} would reach {new_len} tokens; the model has {self.max_seq_len} positions")
         plans = []
         for group in self.groups:
             pages = group.pages[slot]
@@ -178,22 +179,51 @@ class SequenceCache:
             if group.need.window > 0:
                 first_visible = max(0, start - group.need.window + 1)
                 release = [i for i in range(min(first_visible // PAGE_TOKENS, len(pages))) if pages[i] >= 0]
-            want = pages_for(new_len) - len(pages)
-            if want > group.pool.n_free + len(release):
+            plans.append((group, release, max(0, pages_for(new_len) - len(pages))))
+        return plans
+
+    def extend_many(self, slots: Sequence[int], new_tokens: Sequence[int]) -> List[int]:
+        """Make room for `new_tokens[b]` more tokens of `slots[b]`, for all of them or for none: the positions
+        of each sequence's first new token.  Windowed groups first give back the pages that no query of the
+        step can see.  If a sequence would pass the model's positions (IndexError) or a pool runs out
+        (CacheFull), no length and no page has changed."""
+        if len(set(slots)) != len(slots):
+            raise ValueError("a sequence appears twice in one step")
+        plans = [self._plan(slot, n) for slot, n in zip(slots, new_tokens)]
+        for g, group in enumerate(self.groups):
+            want = sum(p[g][2] for p in plans)
+            freed = sum(len(p[g][1]) for p in plans)
+            if want > group.pool.n_free + freed:
                 raise CacheFull(
-                    f"no room for {new_tokens} more tokens of slot {slot}: {want} pages needed, "
-                    f"{group.pool.n_free + len(release)} free of {group.pool.n_pages}"
-                )
-            plans.append((group, release, want))
-        for group, release, want in plans:
-            pages = group.pages[slot]
-            for i in release:
-                group.pool.free(pages[i])
-                pages[i] = -1
-            for _ in range(max(want, 0)):
-                pages.append(group.pool.alloc())
-        self._live[slot] = new_len
-        return start
+                    f"the step needs {want} more cache pages of group {g}, {group.pool.n_free + freed} are free "
+                    f"of {group.pool.n_pages}")
+        starts = []
+        for slot, n, plan in zip(slots, new_tokens, plans):
+            for group, release, _ in plan:
+                pages = group.pages[slot]
+                for i in release:
+                    group.pool.free(pages[i])
+                    pages[i] = -1
+        for slot, n, plan in zip(slots, new_tokens, plans):
+            for group, _, want in plan:
+                pages = group.pages[slot]
+                for _ in range(want):
+                    pages.append(group.pool.alloc())
+            starts.append(self._live[slot])
+            self._live[slot] += n
+            self._clock += 1
+            self._stamp[slot] = self._clock
+        return starts
+
+    def extend(self, slot: int, new_tokens: int) -> int:
+        """Make room for `new_tokens` more tokens of `slot`; returns the position of the first of them.
+        Nothing changes if the room cannot be made."""
+        return self.extend_many([slot], [new_tokens])[0]
+
+    def stamp(self, slot: int) -> int:
+        """A number that changes whenever the slot is handed out or its sequence grows, and never comes back:
+        who remembers it can tell whether the sequence is still as they left it."""
+        return self._stamp[slot]
 
     def block_table(self, group_index: int, slots: Sequence[int], n_columns: Optional[int] = None) -> torch.Tensor:
         """int32 [len(slots), n_columns] page numbers on the host (unused entries and released pages: -1)."""

@@ -74,16 +74,20 @@ def main(argv=None) -> int:
     from ..tokenizers import get_tokenizer
 
     seed = 42 if args.deterministic else args.seed
+    if args.architecture not in ("hf_pretrained", "hf_configured") and args.variant is None:
+        print("--variant is needed with --architecture", args.architecture, file=sys.stderr)
+        return 2
     print("loading model")
-    if args.architecture in ("hf_pretrained", "hf_configured"):
-        model = get_model(args.architecture, model_path=args.model_path or args.variant, device_type=args.device_type,
-                          data_type=args.default_dtype, random_seed=args.random_seed)
-    else:
-        if args.variant is None:
-            print("--variant is needed with --architecture", args.architecture, file=sys.stderr)
-            return 2
-        model = get_model(args.architecture, args.variant, model_path=args.model_path, device_type=args.device_type,
-                          source=args.model_source, data_type=args.default_dtype, random_seed=args.random_seed)
+    try:
+        if args.architecture in ("hf_pretrained", "hf_configured"):
+            model = get_model(args.architecture, model_path=args.model_path or args.variant, device_type=args.device_type,
+                              data_type=args.default_dtype, random_seed=args.random_seed)
+        else:
+            model = get_model(args.architecture, args.variant, model_path=args.model_path, device_type=args.device_type,
+                              source=args.model_source, data_type=args.default_dtype, random_seed=args.random_seed)
+    except (RuntimeError, KeyError, ValueError, FileNotFoundError) as err:  # no GPU, unknown names, a checkpoint that does not fit
+        print(f"could not load the model: {err}", file=sys.stderr)
+        return 1
     tokenizer = get_tokenizer(args.tokenizer)
     print("loading complete")
 
@@ -119,7 +123,7 @@ def main(argv=None) -> int:
     print("==================")
     start = time.time()
     result = generate(model, ids, max_new_tokens=args.max_new_tokens, use_cache=True, do_sample=args.do_sample,
-                      temperature=args.temperature, top_k=args.top_k, max_seq_len=model.config.max_expected_seq_len,
+                      temperature=args.temperature, top_k=args.top_k, max_seq_len=model.spec.max_seq_len,
                       eos_token_id=tokenizer.eos_token_id, extra_kwargs=padding_kwargs, seed=seed)
     elapsed = time.time() - start
     if result.dim() == 1:

@@ -82,8 +82,13 @@ class LLaMAConfig(ModelConfig):
         if self.p_dropout:
             problems.append("p_dropout must be 0: this library only generates")
         kind = (self.rope_scaling or {}).get("rope_type", "regular")
-        if kind not in ("regular", "llama3", "ntk"):
-            problems.append(f"rope_scaling rope_type {kind!r} is not one of regular, llama3, ntk")
+        if kind == "ntk":
+            # fms/modules/positions.py:135-168, 311-355: the table is chosen by the longest sequence of each call, so
+            # a token's rotation depends on how the tokens were cut into calls and on the rest of the batch
+            problems.append("rope_scaling rope_type 'ntk' is not built: its rotation depends on the length of each "
+                            "call, which a step function over a cache cannot reproduce; use regular or llama3")
+        elif kind not in ("regular", "llama3"):
+            problems.append(f"rope_scaling rope_type {kind!r} is not one of regular, llama3")
         if problems:
             raise ValueError("invalid LLaMAConfig: " + "; ".join(problems))
 

@@ -89,6 +89,10 @@ int fmsamd_gemm_f32(const float* a, long lda, const float* w, const float* bias,
                     int K, hipStream_t stream);
 int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const void* bias, int bias_dtype, void* c, int out_dtype,
                      long ldc, int M, int N, int K, hipStream_t stream);
+// The same product for any K and any row stride (the MFMA kernels need multiples of 8): element loads and
+// float32 FMA.  Slow; it exists so that no width a configuration allows is refused.
+int fmsamd_gemm_bf16_any(const void* a, long lda, const void* w, const void* bias, int bias_dtype, void* c,
+                         int out_dtype, long ldc, int M, int N, int K, hipStream_t stream);
 // A row norm left to the product that reads the rows: the rows hold stream * norm weight, and the sums of
 // squares of the stream come as `count` partial sums per row (partials[m * count + i]).  The product is
 // multiplied by rsqrt(sum / K + eps) of its row before the bias.  A null pointer (or null partials): none.

@@ -22,9 +22,12 @@
 #define SG_BN 64
 #define SG_BK 16
 
+// InT float: the true 32-bit product.  InT bf16: the product for sizes the MFMA kernels refuse (K or a row
+// stride that is no multiple of 8, so that rows are not 16-byte aligned): element loads, float32 FMA.
+template <typename InT, typename BiasT, typename OutT>
 __global__ void __launch_bounds__(256)
-    sgemm_nt_kernel(const float* __restrict__ a, long lda, const float* __restrict__ w, const float* __restrict__ bias,
-                    float* __restrict__ c, long ldc, int M, int N, int K) {
+    sgemm_nt_kernel(const InT* __restrict__ a, long lda, const InT* __restrict__ w, const BiasT* __restrict__ bias,
+                    OutT* __restrict__ c, long ldc, int M, int N, int K) {
   __shared__ float as[SG_BK][SG_BM + 1];
   __shared__ float ws[SG_BK][SG_BN + 1];
   const int tx = threadIdx.x % 16;  // n direction
@@ -36,9 +39,9 @@ __global__ void __launch_bounds__(256)
     for (int i = threadIdx.x; i < SG_BM * SG_BK; i += 256) {
       const int row = i / SG_BK, kk = i % SG_BK;
       const int m = m0 + row, k = k0 + kk;
-      as[kk][row] = (m < M && k < K) ? a[(size_t)m * lda + k] : 0.f;
+      as[kk][row] = (m < M && k < K) ? to_f32(a[(size_t)m * lda + k]) : 0.f;
       const int n = n0 + row;
-      ws[kk][row] = (n < N && k < K) ? w[(size_t)n * K + k] : 0.f;
+      ws[kk][row] = (n < N && k < K) ? to_f32(w[(size_t)n * K + k]) : 0.f;
     }
     __syncthreads();
 #pragma unroll
@@ -63,7 +66,7 @@ __global__ void __launch_bounds__(256)
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
-      if (n < N) c[(size_t)m * ldc + n] = acc[i][j] + (bias ? bias[n] : 0.f);
+      if (n < N) c[(size_t)m * ldc + n] = from_f32<OutT>(acc[i][j] + (bias ? to_f32(bias[n]) : 0.f));
     }
   }
 }
@@ -75,8 +78,34 @@ extern "C" int fmsamd_gemm_f32(const float* a, long lda, const float* w, const f
   FMS_REQUIRE(lda >= K && ldc >= N, "gemm_f32: leading dimensions too small");
   dim3 grid(ceil_div(N, SG_BN), ceil_div(M, SG_BM));
   FMS_REQUIRE(grid.y <= 65535, "gemm_f32: M=%d exceeds one launch", M);
-  sgemm_nt_kernel<<<grid, 256, 0, stream>>>(a, lda, w, bias, c, ldc, M, N, K);
+  sgemm_nt_kernel<float, float, float><<<grid, 256, 0, stream>>>(a, lda, w, bias, c, ldc, M, N, K);
   FMS_LAUNCH_CHECK("gemm_f32");
+  return 0;
+}
+
+extern "C" int fmsamd_gemm_bf16_any(const void* a, long lda, const void* w, const void* bias, int bias_dtype, void* c,
+                                    int out_dtype, long ldc, int M, int N, int K, hipStream_t stream) {
+  if (M == 0 || N == 0) return 0;
+  FMS_REQUIRE(M > 0 && N > 0 && K > 0, "gemm_bf16_any: bad sizes M=%d N=%d K=%d", M, N, K);
+  FMS_REQUIRE(lda >= K && ldc >= N, "gemm_bf16_any: leading dimensions too small");
+  dim3 grid(ceil_div(N, SG_BN), ceil_div(M, SG_BM));
+  FMS_REQUIRE(grid.y <= 65535, "gemm_bf16_any: M=%d exceeds one launch", M);
+  const bool fb = bias != nullptr && bias_dtype == FMS_F32;
+#define FMS_SG(B, O)                                                                                                 \
+  sgemm_nt_kernel<bf16, B, O><<<grid, 256, 0, stream>>>((const bf16*)a, lda, (const bf16*)w, (const B*)bias, (O*)c, \
+                                                        ldc, M, N, K)
+  if (out_dtype == FMS_BF16 && !fb)
+    FMS_SG(bf16, bf16);
+  else if (out_dtype == FMS_BF16 && fb)
+    FMS_SG(float, bf16);
+  else if (out_dtype == FMS_F32 && !fb)
+    FMS_SG(bf16, float);
+  else if (out_dtype == FMS_F32 && fb)
+    FMS_SG(float, float);
+  else
+    FMS_REQUIRE(false, "gemm_bf16_any: unknown output dtype %d", out_dtype);
+#undef FMS_SG
+  FMS_LAUNCH_CHECK("gemm_bf16_any");
   return 0;
 }
 

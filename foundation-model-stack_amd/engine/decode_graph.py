@@ -72,6 +72,7 @@ class DecodeGraph:
         self.slots: Tuple[int, ...] = ()
         self.next_tokens: Optional[List[int]] = None  # tokens now in self.tokens (the last step's choices)
         self.n_pages: List[int] = []
+        self.stamps: List[int] = []  # the cache's stamp of every sequence after the last replay
         self.graph: Optional[torch.cuda.CUDAGraph] = None
 
     def _run(self) -> None:
@@ -83,7 +84,7 @@ class DecodeGraph:
     def capture(self) -> None:
         # Padding rows only (sequence -1): nothing is written to the cache while warming up and capturing.
         self.seq_of_token.fill_(-1)
-        self.slots, self.next_tokens = (), None
+        self.slots, self.next_tokens, self.stamps = (), None, []
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):

@@ -15,7 +15,7 @@ import torch
 
 import os
 
-from ..cache import CacheFull, pages_for
+from ..cache import pages_for
 from ..sampling import SamplingParams, choose
 from .batch import StepBatch, build_batch
 from .decode_graph import CONTEXT_HEADROOM, DecodeGraph, context_bucket, row_bucket
@@ -92,15 +92,10 @@ class Engine:
         for t in tokens:
             if not 0 <= t < self.vocab:
                 raise IndexError(f"token id {t} is outside the vocabulary of {self.vocab}")
-        for group in self.cache.groups:
-            if group.need.window == 0:
-                need = sum(1 for s in slots if self.cache.length(s) % 64 == 0)
-                if need > group.pool.n_free:
-                    raise CacheFull(f"the step needs {need} more cache pages, {group.pool.n_free} are free")
-        for s in slots:
-            if self.cache.length(s) + 1 > self.cache.max_seq_len:
-                raise IndexError(f"sequence in slot {s} has reached the model's {self.cache.max_seq_len} positions")
-        positions = [self.cache.extend(s, 1) for s in slots]
+        # what the sequences looked like before this step: a graph's buffers still describe them only if
+        # nothing but the graph's own last replay has touched them since
+        before = [self.cache.stamp(s) for s in slots]
+        positions = self.cache.extend_many(slots, [1] * len(slots))  # room for all, or for none
         rows = row_bucket(len(slots))
         longest = max(positions) + 1
         how = (sampling.do_sample, float(sampling.temperature), int(sampling.top_k or 0))
@@ -114,10 +109,11 @@ class Engine:
             graph = self._graphs[(rows, ctx) + how] = DecodeGraph(self, rows, ctx, sampling)
             graph.capture()
             self.graph_captures.append((rows, ctx))
-        if graph.slots == tuple(slots) and graph.next_tokens == tokens:
-            graph.refresh_pages()
+        if graph.slots == tuple(slots) and graph.stamps == before and graph.next_tokens == tokens:
+            graph.refresh_pages()  # the same sequences, one step on, fed what the graph chose: its buffers are current
         else:
             graph.load(slots, tokens, positions, seeds or [0] * len(slots), counters or [0] * len(slots))
+        graph.stamps = [self.cache.stamp(s) for s in slots]
         return graph.replay()
 
     def prepare(self, slots, tokens, want) -> StepBatch:
@@ -138,16 +134,11 @@ class Engine:
             want = [list(range(len(t))) for t in tokens]
         elif len(want) != len(slots):
             raise ValueError("one list of wanted places per sequence is needed")
-        # room for all, or for none
-        for group in self.cache.groups:
-            if group.need.window == 0:
-                need = sum(max(0, pages_for(self.cache.length(s) + len(t)) - len(group.pages[s])) for s, t in zip(slots, tokens))
-                if need > group.pool.n_free:
-                    raise CacheFull(f"the step needs {need} more cache pages, {group.pool.n_free} are free")
-        for s, t in zip(slots, tokens):
-            if self.cache.length(s) + len(t) > self.cache.max_seq_len:
-                raise IndexError(f"sequence in slot {s} would reach {self.cache.length(s) + len(t)} tokens; the model has {self.cache.max_seq_len} positions")
-        starts = [self.cache.extend(s, len(t)) for s, t in zip(slots, tokens)]
+        for b, (w, t) in enumerate(zip(want, tokens)):
+            for place in w:
+                if not 0 <= int(place) < len(t):
+                    raise IndexError(f"wanted place {place} is outside the {len(t)} tokens of sequence {b}")
+        starts = self.cache.extend_many(slots, [len(t) for t in tokens])  # room for all, or for none
         n_tokens = sum(len(t) for t in tokens)
         sizes = set()
         if any(len(t) > 1 for t in tokens):

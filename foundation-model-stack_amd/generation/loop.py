@@ -139,45 +139,6 @@ def generate_requests(
 # --------------------------------------------------------------------------
 # the reference's call
 # --------------------------------------------------------------------------
-def pad_input_ids(input_ids_list: List[torch.Tensor], min_pad_length: int = 0, is_causal_mask=True,
-                  padding_side="left", position_ids_offset=0, pad_token_id=0):
-    """A rectangular tensor from prompts of unequal lengths, with the mask and position_ids the
-    reference builds (fms/utils/generation.py:16-109).  ``generate`` reads the real lengths back
-    from ``position_ids``/``mask``; the engine itself never sees padding."""
-    max_len = max([min_pad_length] + [seq.size(0) for seq in input_ids_list])
-    rows, masks, positions = [], [], []
-    for seq in input_ids_list:
-        n = seq.size(0)
-        pads = torch.full((max_len - n,), pad_token_id, dtype=torch.long, device=seq.device)
-        real = torch.ones(n, dtype=torch.bool, device=seq.device)
-        fake = torch.zeros(max_len - n, dtype=torch.bool, device=seq.device)
-        pos_pad = torch.zeros(max_len - n, dtype=torch.long, device=seq.device)
-        pos = torch.arange(0, n, dtype=torch.long, device=seq.device)
-        if padding_side == "left":
-            rows.append(torch.cat((pads, seq)))
-            masks.append(torch.cat((fake, real)))
-            positions.append(torch.cat((pos_pad, pos)))
-        elif padding_side == "right":
-            rows.append(torch.cat((seq, pads)))
-            masks.append(torch.cat((real, fake)))
-            positions.append(torch.cat((pos, pos_pad)))
-        else:
-            raise NotImplementedError("padding_side must be 'right' or left'")
-    input_ids = torch.stack(rows)
-    mask = torch.stack(masks)
-    mask = mask.unsqueeze(-1) == mask.unsqueeze(-2)
-    if is_causal_mask:
-        mask = mask.tril()
-    mask = torch.where(mask.logical_not(), -torch.inf, 0.0)
-    position_ids = torch.stack(positions) + position_ids_offset
-    return input_ids, {
-        "mask": mask,
-        "position_ids": position_ids,
-        "lengths": [seq.size(0) for seq in input_ids_list],
-        "padding_side": padding_side,
-    }
-
-
 def _real_tokens(input_ids: torch.Tensor, extra_kwargs) -> List[List[int]]:
     """Rows of a rectangular batch without their padding.
 
@@ -293,25 +254,3 @@ def default_engine(model, prompts, max_new_tokens):
         engine = Engine(model, max_tokens=need, max_slots=max(len(prompts), 1))
         model._default_engine = engine
     return engine
-
-
-def truncate_after_eos(result: torch.Tensor, eos_token_id) -> torch.Tensor:
-    """Cut a 1-D result after its first eos token (fms/utils/generation.py:372-387)."""
-    if eos_token_id is None:
-        return result
-    idx = torch.where(result == eos_token_id)[0]
-    if idx.shape[0] >= 1:
-        result = result[: idx[0] + 1]
-    return result
-
-
-def trim_prefix(result: torch.Tensor, pad_token_id: int = 0) -> torch.Tensor:
-    """Drop leading pad tokens and the token that follows them... as the reference does
-    (fms/utils/generation.py:390-413): everything up to and including the last leading pad."""
-    if result[0] != pad_token_id:
-        return result
-    diff = (result != pad_token_id).diff()
-    first = torch.where(diff > 0)[0]
-    if first.numel() == 0:
-        return result
-    return result[first[0] + 1 :]

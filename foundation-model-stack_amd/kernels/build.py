@@ -20,6 +20,7 @@ from typing import List, Optional
 
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 LIB_NAME = "libfmsamd.so"
+DIGEST_NAME = "digest.txt"
 ARCH = "gfx950"
 
 # -packed-fp32-ops: keep the compiler from forming packed float32 instructions.
@@ -98,8 +99,11 @@ def build(verbose: bool = True) -> str:
     start = time.time()
     _say(f"compiling {len(srcs)} HIP sources for {ARCH} into {out_dir}", verbose)
 
+    # objects go to a folder of this process, so that two processes building at once do not write one file
+    obj_dir = tempfile.mkdtemp(prefix=f".obj{os.getpid()}_", dir=out_dir)
+
     def compile_one(src: str) -> str:
-        obj = os.path.join(out_dir, os.path.basename(src)[:-4] + ".o")
+        obj = os.path.join(obj_dir, os.path.basename(src)[:-4] + ".o")
         cmd = [hipcc, *HIPCC_FLAGS, "-I", CSRC, "-c", src, "-o", obj]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0:
@@ -107,34 +111,53 @@ def build(verbose: bool = True) -> str:
         _say(f"compiled {os.path.basename(src)} ({time.time() - start:.0f} s)", verbose)
         return obj
 
-    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
-        objs = list(pool.map(compile_one, srcs))
-    tmp = os.path.join(out_dir, f".{LIB_NAME}.{os.getpid()}")
-    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp]
-    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    if proc.returncode != 0:
-        raise RuntimeError(f"hipcc failed to link:\n{proc.stdout}")
-    lib = os.path.join(out_dir, LIB_NAME)
-    os.replace(tmp, lib)
-    with open(os.path.join(out_dir, "digest.txt"), "w") as f:
-        f.write(source_digest())
+    try:
+        digest = source_digest()
+        with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+            objs = list(pool.map(compile_one, srcs))
+        tmp = os.path.join(obj_dir, LIB_NAME)
+        cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp]
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise RuntimeError(f"hipcc failed to link:\n{proc.stdout}")
+        lib = os.path.join(out_dir, LIB_NAME)
+        os.replace(tmp, lib)
+        digest_tmp = os.path.join(obj_dir, DIGEST_NAME)
+        with open(digest_tmp, "w") as f:
+            f.write(digest)
+        os.replace(digest_tmp, os.path.join(out_dir, DIGEST_NAME))
+    finally:
+        shutil.rmtree(obj_dir, ignore_errors=True)
     _say(f"linked {lib} ({time.time() - start:.0f} s)", verbose)
     return lib
 
 
+def library_is_current(lib: str) -> bool:
+    """True if the library's folder records the digest of the sources as they are now."""
+    try:
+        with open(os.path.join(os.path.dirname(lib), DIGEST_NAME)) as f:
+            return f.read().strip() == source_digest()
+    except OSError:
+        return False
+
+
 def ensure_built(verbose: bool = True) -> str:
-    """The path of a built library; builds only when none is there."""
-    lib = find_library()
-    if lib is not None:
-        digest_file = os.path.join(os.path.dirname(lib), "digest.txt")
-        try:
-            with open(digest_file) as f:
-                if f.read().strip() != source_digest():
-                    _say(f"{lib} is older than the sources; call build() to refresh it", verbose)
-        except OSError:
-            pass
-        return lib
-    return build(verbose)
+    """The path of a library built from the sources as they are now.  A built copy whose recorded digest
+    matches is used as it is; otherwise the library is compiled.  A copy that is older than the sources is
+    never used: if it cannot be replaced (no compiler, no writable folder) this raises."""
+    for folder in build_dirs():
+        lib = os.path.join(folder, LIB_NAME)
+        if os.path.isfile(lib) and library_is_current(lib):
+            return lib
+    stale = find_library()
+    if stale is not None:
+        _say(f"{stale} was built from other sources than the present ones: compiling again", verbose)
+    try:
+        return build(verbose)
+    except Exception as err:
+        if stale is not None:
+            raise RuntimeError(f"{stale} does not match the present sources and could not be rebuilt: {err}") from err
+        raise
 
 
 if __name__ == "__main__":

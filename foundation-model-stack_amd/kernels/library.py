@@ -39,6 +39,7 @@ _SIGNATURES = {
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
     "fmsamd_gemm_f32": [P, L, P, P, P, L, I, I, I, P],
     "fmsamd_gemm_bf16": [P, L, P, P, I, P, I, L, I, I, I, P],
+    "fmsamd_gemm_bf16_any": [P, L, P, P, I, P, I, L, I, I, I, P],
     "fmsamd_gemm_skinny_workspace": [I, I, I],
     "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P, P, L, P],
     "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P, P, L, P],
@@ -67,7 +68,7 @@ def load(verbose: bool = True) -> ctypes.CDLL:
         except Exception as err:  # no compiler, no writable folder, broken library
             raise KernelLibraryMissing(
                 f"the HIP kernel library of fms_amd could not be built or loaded ({err}); "
-                "there is no fallback path: build it with `python -c 'import __graft_entry__ as g; g.build()'`"
+                "there is no fallback path: build it with `python -m fms_amd.kernels.build` (needs hipcc)"
             ) from err
         lib.fmsamd_last_error.restype = c_char_p
         lib.fmsamd_last_error.argtypes = []

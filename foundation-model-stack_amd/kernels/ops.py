@@ -467,9 +467,17 @@ def linear(
         raise TypeError(f"weights are float32 or bfloat16, not {weight.dtype}")
     if x.dtype != torch.bfloat16:
         raise TypeError("a bfloat16 weight takes bfloat16 activations")
-    if K % 8 or x.stride(0) % 8:
-        raise ValueError(f"bfloat16 products need K (={K}) and the row stride (={x.stride(0)}) to be multiples of 8")
     bcode = _code(bias.dtype) if bias is not None else 0
+    if K % 8 or x.stride(0) % 8:
+        # rows that are not 16-byte aligned: the element-wise kernel, so that no width is refused
+        if row_norm is not None:
+            raise ValueError("a deferred row norm goes with K and a row stride that are multiples of 8")
+        out = torch.empty(M, N, dtype=out_dtype, device=x.device)
+        for m0 in range(0, M, 65535 * 64):
+            m = min(65535 * 64, M - m0)
+            check(lib.fmsamd_gemm_bf16_any(x[m0:].data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), bcode,
+                                           out[m0:].data_ptr(), _code(out_dtype), out.stride(0), m, N, K, _stream()))
+        return out
     if M <= SKINNY_FAST_ROWS or (M <= SKINNY_MAX_ROWS and not (allow_library and out_dtype == torch.bfloat16)):
         out = torch.empty(M, N, dtype=out_dtype, device=x.device)
         ws, ws_bytes = _skinny_workspace(M, N, K, x.device)
@@ -538,14 +546,13 @@ def gated_linear(
     if weight.shape[0] % 2:
         raise ValueError("the stacked gate/up weight needs an even number of rows")
     hidden = weight.shape[0] // 2
-    if x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M <= (SKINNY_FAST_ROWS if allow_library else SKINNY_MAX_ROWS):
+    if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M <= (SKINNY_FAST_ROWS if allow_library else SKINNY_MAX_ROWS)
+            and x.dim() == 2 and x.shape[1] % 8 == 0 and x.stride(0) % 8 == 0):
         _need_cuda(x, weight, bias)
         _rows2d("x", x)
         K = x.shape[1]
         if weight.shape[1] != K or not weight.is_contiguous():
             raise ValueError("weight must be contiguous [2*hidden, K] with K the width of x")
-        if K % 8 or x.stride(0) % 8:
-            raise ValueError(f"bfloat16 products need K (={K}) and the row stride to be multiples of 8")
         if bias is not None and (bias.shape != (2 * hidden,) or not bias.is_contiguous()):
             raise ValueError(f"bias must be a contiguous [{2 * hidden}] tensor")
         out = torch.empty(M, hidden, dtype=torch.bfloat16, device=x.device)

@@ -17,7 +17,6 @@ from typing import Optional, Union
 import torch
 
 from .architectures import architecture_for_hf, get_architecture, variant_config
-from .architectures.llama import detect_source
 from .config import ModelConfig
 from .engine.model import DecoderModel
 from .weights import Checkpoint, init_random, load_checkpoint, random_tensor, write_safetensors
@@ -91,6 +90,9 @@ def get_model(
     device = torch.device(device_type if ":" in str(device_type) or device_type != "cuda" else "cuda:0")
     if device.type != "cuda":
         raise RuntimeError("fms_amd models run on the GPU only (device_type='cuda'); there is no CPU path")
+    if not torch.cuda.is_available():  # before anything is allocated: the message is this library's, not the runtime's
+        raise RuntimeError("fms_amd models run on an AMD GPU, and this machine shows none to PyTorch "
+                           "(torch.cuda.is_available() is False); there is no CPU path")
 
     ckpt_dtype = None
     if model_path is not None:
@@ -98,7 +100,9 @@ def get_model(
         try:
             names = ckpt.keys()
             if source is None:
-                source = detect_source(names)
+                if arch.detect_source is None:
+                    raise ValueError(f"architecture {arch.name} cannot tell a checkpoint's source from its tensor names: pass source=")
+                source = arch.detect_source(names)
             floats = [ckpt.stored_dtype(n) for n in names if ckpt.stored_dtype(n).is_floating_point]
             if floats:
                 ckpt_dtype = torch.float32 if all(d in (torch.float32, torch.float64) for d in floats) else torch.bfloat16
@@ -111,7 +115,7 @@ def get_model(
     model = DecoderModel(arch.build_spec(config), dtype, config=config)
     model.architecture = arch.name
     if model_path is not None:
-        load_checkpoint(model, model_path, arch.name, source, device)
+        load_checkpoint(model, model_path, arch.name, source, device, forced_dtype=data_type is not None)
     else:
         init_random(model, random_seed, device)
     model.finalize_all(device)

@@ -74,7 +74,8 @@ class MultiHeadAttention(Mixer):
         """True if projection, rotation and cache write of this step run as one kernel."""
         rotates_by_table = self.position_encoder is None or self.position_encoder.rotary_tables() is not None
         return (batch.is_decode and rows <= ops.QKV_ROPE_MAX_ROWS and dtype == torch.bfloat16
-                and self.qkv.w["weight"].dtype == torch.bfloat16 and self.head_dim % 16 == 0 and rotates_by_table)
+                and self.qkv.w["weight"].dtype == torch.bfloat16 and self.head_dim % 16 == 0 and self.width % 8 == 0
+                and rotates_by_table)
 
     def accepts_normed_rows(self, rows: int, dtype, batch) -> bool:
         return self._fused_decode(rows, dtype, batch)

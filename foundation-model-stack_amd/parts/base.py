@@ -18,7 +18,9 @@ import torch
 class ParamSpec:
     shape: Tuple[int, ...]
     init: str = "normal"  # "normal" (std 0.02), "ones", "zeros": what random-weights mode writes
-    kind: str = "float"  # "float": model dtype unless the file stores 32-bit; "int": int32
+    # "float": the model's type; "scale": a norm's scale or shift, which stays 32-bit if the file stores it so;
+    # "int": int32
+    kind: str = "float"
 
 
 class Part:

@@ -28,9 +28,9 @@ class ParameterizedNorm(Part):
         super().__init__()
         self.width, self.eps, self.use_mean = width, float(eps), use_mean
         if elementwise_scale:
-            self.declare("weight", (width,), init="ones")
+            self.declare("weight", (width,), init="ones", kind="scale")
         if elementwise_shift:
-            self.declare("bias", (width,), init="zeros")
+            self.declare("bias", (width,), init="zeros", kind="scale")
 
     def add_norm(
         self,

@@ -10,33 +10,38 @@ from typing import List
 
 
 class CharTokenizer:
+    """A character is the token of its code point: 256 tokens, code points from 256 on become token 0;
+    token 2 begins a text and token 3 ends it (the ASCII controls of those names)."""
+
     bos_token_id = 2
     eos_token_id = 3
-
-    def tokenize(self, text: str) -> List[str]:
-        return list(text)
-
-    def convert_tokens_to_ids(self, tokens) -> List[int]:
-        if isinstance(tokens, str):
-            if len(tokens) != 1:
-                raise RuntimeError("Only single character str tokens can be converted using the CharTokenizer.")
-            return ord(tokens) if ord(tokens) < 256 else 0
-        return [ord(t) if len(t) == 1 and ord(t) < 256 else 0 for t in tokens]
-
-    def convert_ids_to_tokens(self, ids) -> List[str]:
-        return [chr(int(i)) for i in ids]
-
-    def convert_tokens_to_string(self, tokens: List[str]) -> str:
-        return "".join(tokens)
-
-    def encode(self, text: str) -> List[int]:
-        return self.convert_tokens_to_ids(self.tokenize(text))
-
-    def decode(self, ids) -> str:
-        return self.convert_tokens_to_string(self.convert_ids_to_tokens(ids))
+    _SIZE = 256
 
     def vocab_size(self) -> int:
-        return 256
+        return self._SIZE
+
+    def encode(self, text: str) -> List[int]:
+        return [code if code < self._SIZE else 0 for code in map(ord, text)]
+
+    def decode(self, ids) -> str:
+        return "".join(map(chr, map(int, ids)))
+
+    # the reference's older four-call interface (tests/utils/test_generate.py uses it)
+    def tokenize(self, text: str) -> List[str]:
+        return [c for c in text]
+
+    def convert_tokens_to_ids(self, tokens):
+        if isinstance(tokens, str):  # one token gives one id, as the reference's other tokenizers do
+            if len(tokens) != 1:
+                raise RuntimeError(f"a token of the character tokenizer is one character, got {tokens!r}")
+            return self.encode(tokens)[0]
+        return [self.encode(t)[0] if len(t) == 1 else 0 for t in tokens]
+
+    def convert_ids_to_tokens(self, ids) -> List[str]:
+        return list(self.decode(ids))
+
+    def convert_tokens_to_string(self, tokens) -> str:
+        return "".join(tokens)
 
 
 class _SentencePiece:

@@ -1,8 +1,12 @@
 """Filling a model's parameters: from a checkpoint by tensor name, or at random from a seed.
 
-Kept types: floating tensors become the model's type (bfloat16 or float32),
-except that a tensor the checkpoint stores in 32-bit stays 32-bit; integer
-tensors become int32.  Every problem of a checkpoint — tensors the model lacks,
+Kept types.  With a type asked for (``data_type``), floating tensors are cast
+to it, as the reference does (fms/utils/serialization.py:679-687,
+tests/models/test_getmodel_datatype.py:58-90); only norm scales and shifts
+(parameters of kind "scale") that the file stores in 32-bit stay 32-bit: the
+norm kernels compute in 32-bit and read either type.  With no type asked for,
+the model runs in the checkpoint's type, and in a bfloat16 model a tensor that
+the file stores in 32-bit stays 32-bit.  Integer tensors become int32.  Every problem of a checkpoint — tensors the model lacks,
 tensors the model has and the checkpoint lacks, wrong shapes — is collected and
 raised as one error.  (The reference warns about unused keys and leaves missing
 ones uninitialised, fms/utils/serialization.py:604-608, fms/models/__init__.py:494-501;
@@ -35,11 +39,12 @@ class WeightsError(ValueError):
         super().__init__("\n".join(lines))
 
 
-def kept_dtype(stored: torch.dtype, kind: str, model_dtype: torch.dtype) -> torch.dtype:
+def kept_dtype(stored: torch.dtype, kind: str, model_dtype: torch.dtype, forced: bool = False) -> torch.dtype:
+    """The type in which a checkpoint tensor is kept on the device.  forced: the caller asked for model_dtype."""
     if kind == "int" or not stored.is_floating_point:
         return torch.int32
-    if stored in (torch.float32, torch.float64) and model_dtype == torch.bfloat16:
-        return torch.float32  # a tensor stored in 32-bit stays so
+    if stored in (torch.float32, torch.float64) and model_dtype == torch.bfloat16 and (kind == "scale" or not forced):
+        return torch.float32  # stored in 32-bit and nobody asked otherwise: it stays so
     return model_dtype
 
 
@@ -57,8 +62,10 @@ def _layer_groups(names: List[str]) -> List[List[str]]:
     return [groups[k] for k in sorted(groups)]
 
 
-def load_checkpoint(model, path: str, architecture: str, source: Optional[str], device, verbose: bool = False) -> None:
-    """Bind every parameter of `model` from the checkpoint at `path`; one WeightsError lists all that is wrong."""
+def load_checkpoint(model, path: str, architecture: str, source: Optional[str], device, verbose: bool = False,
+                    forced_dtype: bool = False) -> None:
+    """Bind every parameter of `model` from the checkpoint at `path`; one WeightsError lists all that is wrong.
+    forced_dtype: the model's type was asked for by the caller, so floating tensors are cast to it."""
     ckpt = Checkpoint(path, source)
     try:
         adapter = get_adapter(architecture, source)
@@ -74,7 +81,7 @@ def load_checkpoint(model, path: str, architecture: str, source: Optional[str], 
                 if tuple(tensor.shape) != spec.shape:
                     wrong.append((name, tuple(tensor.shape), spec.shape))
                     continue
-                dtype = kept_dtype(tensor.dtype, spec.kind, model.dtype)
+                dtype = kept_dtype(tensor.dtype, spec.kind, model.dtype, forced_dtype)
                 part.bind(local, tensor.to(dtype).contiguous().to(device))
                 bound.add(name)
             del partial

@@ -203,6 +203,12 @@ def test_kept_dtypes():
     assert kept_dtype(torch.float32, "float", torch.bfloat16) == torch.float32  # stored in 32-bit: stays so
     assert kept_dtype(torch.bfloat16, "float", torch.float32) == torch.float32
     assert kept_dtype(torch.int64, "int", torch.bfloat16) == torch.int32
+    # a type that the caller asked for is what floating tensors get (tests/models/test_getmodel_datatype.py:58-90) ...
+    assert kept_dtype(torch.float32, "float", torch.bfloat16, forced=True) == torch.bfloat16
+    assert kept_dtype(torch.bfloat16, "float", torch.float32, forced=True) == torch.float32
+    # ... except a norm's scale, which the kernels read in either type
+    assert kept_dtype(torch.float32, "scale", torch.bfloat16, forced=True) == torch.float32
+    assert kept_dtype(torch.bfloat16, "scale", torch.bfloat16, forced=True) == torch.bfloat16
 
 
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
@@ -244,6 +250,44 @@ def test_loading_keeps_types_and_ties_the_head(tmp_path):
     model32 = DecoderModel(llama_spec(config), torch.float32, config=config)
     load_checkpoint(model32, folder, "llama", "hf", "cpu")
     assert model32.layers[1].feed_forward.w2.w["weight"].dtype == torch.float32
+
+
+def test_a_forced_type_casts_what_the_file_stores_in_32_bit(tmp_path):
+    """tests/models/test_getmodel_datatype.py: a checkpoint in 32-bit loaded with data_type bf16 gives a bfloat16
+    model (every linear takes the bfloat16 kernels); with no type given the stored type is kept."""
+    config = LLaMAConfig(**TINY)
+    folder = fms_amd.write_model_folder(str(tmp_path / "m"), config, seed=2, data_type="float32")
+    forced = DecoderModel(llama_spec(config), torch.bfloat16, config=config)
+    load_checkpoint(forced, folder, "llama", "hf", "cpu", forced_dtype=True)
+    for name, spec, part, local in forced.named_specs():
+        want = torch.float32 if spec.kind == "scale" else torch.bfloat16
+        assert part.w[local].dtype == want, name
+    assert forced.layers[0].mixer.dense.streams(4, torch.bfloat16)
+    kept = DecoderModel(llama_spec(config), torch.bfloat16, config=config)
+    load_checkpoint(kept, folder, "llama", "hf", "cpu")
+    assert all(part.w[local].dtype == torch.float32 for _, _, part, local in kept.named_specs())
+    assert not kept.layers[0].mixer.dense.streams(4, torch.bfloat16)
+
+
+def test_the_architecture_tells_a_checkpoints_source():
+    from fms_amd.architectures import get_architecture
+
+    arch = get_architecture("llama")
+    assert arch.detect_source(["model.layers.0.self_attn.q_proj.weight"]) == "hf"
+    assert arch.detect_source(["tok_embeddings.weight", "layers.0.attention.wq.weight"]) == "meta"
+    assert arch.detect_source(["base_model.layers.0.attn.in_proj.query.weight"]) == "fms_unfused"
+    assert arch.detect_source(["base_model.layers.0.attn.in_proj.qkv_fused.weight"]) == "fms"
+    import fms_amd.models as models
+
+    assert not hasattr(models, "detect_source")  # the generic loader asks the architecture
+
+
+def test_ntk_scaling_is_refused_with_the_configuration():
+    """fms/modules/positions.py:135-168: the table depends on the length of each call."""
+    with pytest.raises(ValueError, match="ntk"):
+        LLaMAConfig(**TINY, rope_scaling={"rope_type": "ntk"})
+    with pytest.raises(ValueError, match="ntk"):
+        LLaMAConfig.from_hf_dict({**LLaMAConfig(**TINY).to_hf_dict(), "rope_scaling": {"rope_type": "ntk"}})
 
 
 def test_schedule_is_data():
@@ -339,6 +383,43 @@ def test_cache_groups_and_window_pages():
     cache.free_slot(s)
     cache.check()
     assert cache.groups[1].pool.n_free == 8
+
+
+def test_a_step_that_cannot_be_made_changes_nothing():
+    """Room for all or for none, across groups (one of them windowed) and across the sequences of a step."""
+    kv = [(0, KVNeed(2, 16, 0)), (1, KVNeed(2, 16, 128))]
+    cache = SequenceCache(kv, [], 64 * 8, 4, 2000, device=None)
+    a, b, c = cache.alloc_slot(), cache.alloc_slot(), cache.alloc_slot()
+    assert cache.extend_many([a, b, c], [200, 100, 64]) == [0, 0, 0]  # 4 + 2 + 1 pages in both groups
+    assert cache.extend_many([a], [1]) == [200]  # the window lets go of a's first page: 7 of 8 held there, 7 in full
+    cache.check()
+
+    def snapshot():
+        return ({s: cache.length(s) for s in cache.live_slots()}, [g.pool.n_free for g in cache.groups],
+                [{s: list(p) for s, p in g.pages.items()} for g in cache.groups], [cache.stamp(s) for s in (a, b, c)])
+
+    before = snapshot()
+    with pytest.raises(CacheFull):  # b and c want a page each, the full group has one
+        cache.extend_many([a, b, c], [1, 30, 1])
+    assert snapshot() == before
+    with pytest.raises(IndexError):  # c would pass the model's positions; a and b come first and must not grow
+        cache.extend_many([a, b, c], [1, 1, 3000])
+    assert snapshot() == before
+    with pytest.raises(ValueError):
+        cache.extend_many([a, a], [1, 1])
+    assert snapshot() == before
+    assert cache.pages_needed(b, 30) == 1 and cache.pages_needed(a, 1) == 0
+    assert cache.extend_many([b, a], [30, 1]) == [100, 201]
+    cache.check()
+    # a stamp changes with every growth and with every hand-out, and never repeats
+    stamps = {cache.stamp(a)}
+    cache.extend(a, 1)
+    stamps.add(cache.stamp(a))
+    cache.free_slot(a)
+    again = cache.alloc_slot()
+    assert again == a
+    stamps.add(cache.stamp(again))
+    assert len(stamps) == 3
 
 
 def test_block_table_rows_follow_the_step_order():
@@ -488,6 +569,85 @@ def test_padding_helpers_follow_the_reference():
     assert trim_prefix(torch.tensor([1, 2, 3, 4, 0, 1])).tolist() == [1, 2, 3, 4, 0, 1]
 
 
+def test_padding_helpers_reference_vectors():
+    """tests/utils/test_generate.py:148-198 (the mask as the reference's test builds it) and :289-323
+    (a pad token that is not zero)."""
+    prompts = [torch.arange(1, 5), torch.arange(1, 10)]
+    for min_pad, pads in ((0, (5, 0)), (64, (60, 55))):
+        ids, extra = pad_input_ids(prompts, min_pad_length=min_pad)
+        assert ids.dtype == torch.long and extra["position_ids"].dtype == torch.long
+        assert ids.tolist() == [[0] * pads[0] + list(range(1, 5)), [0] * pads[1] + list(range(1, 10))]
+        assert extra["position_ids"].tolist() == [[0] * pads[0] + list(range(4)), [0] * pads[1] + list(range(9))]
+        is_pad = torch.tensor([[1] * pads[0] + [0] * 4, [1] * pads[1] + [0] * 9], dtype=torch.bool)
+        expected = (is_pad.unsqueeze(-1) == is_pad.unsqueeze(-2)).tril()
+        expected = torch.where(expected.logical_not(), -torch.inf, 0.0)
+        torch.testing.assert_close(extra["mask"], expected)
+    _, extra = pad_input_ids(prompts, min_pad_length=12, pad_token_id=100256)
+    for b, n in enumerate((4, 9)):
+        first = 12 - n
+        for q in range(first, 12):
+            assert (extra["mask"][b, q] == 0).nonzero().flatten().tolist() == list(range(first, q + 1))
+        for q in range(first):
+            assert extra["mask"][b, q, q] == 0
+    ids, extra = pad_input_ids(prompts, padding_side="right", position_ids_offset=3, is_causal_mask=False)
+    assert ids[0].tolist() == [1, 2, 3, 4, 0, 0, 0, 0, 0] and extra["position_ids"][0].tolist() == [3, 4, 5, 6, 3, 3, 3, 3, 3]
+    assert (extra["mask"][0, 0] == 0).nonzero().flatten().tolist() == [0, 1, 2, 3]
+    with pytest.raises(NotImplementedError):
+        pad_input_ids(prompts, padding_side="middle")
+    # tests/utils/test_generate.py:139-145, :281-286
+    result = torch.ones(20)
+    result[10] = 5
+    assert truncate_after_eos(result, 5).tolist() == [1.0] * 10 + [5.0]
+    sentence = torch.cat((torch.zeros(10), torch.ones(20)))
+    assert trim_prefix(sentence).tolist() == [1.0] * 20 and trim_prefix(sentence, pad_token_id=2).tolist() == sentence.tolist()
+    assert trim_prefix(torch.zeros(4)).tolist() == [0.0] * 4
+
+
+def test_char_tokenizer():
+    """fms/utils/tokenizers.py:97-143 and tests/utils/test_generate.py:33-50: a character is its code point."""
+    from fms_amd.tokenizers import CharTokenizer, get_tokenizer
+
+    tok = get_tokenizer("char_tokenizer")
+    assert isinstance(tok, CharTokenizer) and tok.vocab_size() == 256 and (tok.bos_token_id, tok.eos_token_id) == (2, 3)
+    assert tok.encode("AB é\u4e2d") == [65, 66, 32, 233, 0]
+    assert tok.decode([65, 66, 67]) == "ABC"
+    ids = tok.convert_tokens_to_ids(tok.tokenize("ABCDE"))
+    assert ids == [65, 66, 67, 68, 69] and tok.convert_tokens_to_ids("A") == 65
+    assert tok.convert_tokens_to_string(tok.convert_ids_to_tokens(torch.tensor(ids))) == "ABCDE"
+    with pytest.raises(RuntimeError):
+        tok.convert_tokens_to_ids("AB")
+    with pytest.raises(RuntimeError):
+        get_tokenizer("/no/such/tokenizer")
+
+
+def test_command_line_refusals(capsys):
+    """scripts/inference.py:23-113: the reference's option names; what this library cannot do is refused with 2
+    before anything is loaded, and a machine without a GPU gets this library's own words."""
+    from fms_amd.cli.inference import build_parser, main
+
+    options = {a.dest for a in build_parser()._actions}
+    assert {"device_type", "architecture", "variant", "model_path", "model_source", "tokenizer", "no_use_cache",
+            "unfuse_weights", "default_dtype", "compile", "compile_mode", "deterministic", "distributed", "batch_input",
+            "min_pad_length", "attn_name", "context_file"} <= options
+    base = ["--tokenizer", "char_tokenizer"]
+    assert main(base + ["--variant", "micro", "--distributed"]) == 2
+    assert "one process on one GPU" in capsys.readouterr().err
+    assert main(base + ["--variant", "micro", "--default_dtype", "fp16"]) == 2
+    assert "bf16 or fp32" in capsys.readouterr().err
+    assert main(base + ["--variant", "micro", "--attn_name", "sdpa_bidirectional"]) == 2
+    capsys.readouterr()
+    assert main(base) == 2  # --architecture llama without a variant
+    assert "--variant is needed" in capsys.readouterr().err
+    with pytest.raises(SystemExit):  # --tokenizer is required, as in the reference
+        main(["--variant", "micro"])
+    capsys.readouterr()
+    if not torch.cuda.is_available():
+        assert main(base + ["--variant", "micro"]) == 1
+        assert "shows none to PyTorch" in capsys.readouterr().err
+        assert main(base + ["--variant", "no-such-variant"]) == 1
+        assert "not a registered variant" in capsys.readouterr().err
+
+
 def test_sampling_uniforms_are_a_function_of_seed_and_counter():
     from fms_amd.sampling import SamplingParams, request_seed, uniform
 
@@ -502,8 +662,10 @@ def test_sampling_uniforms_are_a_function_of_seed_and_counter():
 def test_no_gpu_means_a_loud_failure():
     if torch.cuda.is_available():
         pytest.skip("this machine has a GPU")
-    with pytest.raises(RuntimeError):
+    with pytest.raises(RuntimeError, match="no CPU path"):
         fms_amd.get_model("llama", "micro", device_type="cpu")
+    with pytest.raises(RuntimeError, match="shows none to PyTorch"):  # this library's words, before any allocation
+        fms_amd.get_model("llama", "micro", device_type="cuda")
     from fms_amd.kernels import ops
 
     with pytest.raises(RuntimeError, match="no CPU fallback"):
@@ -513,6 +675,37 @@ def test_no_gpu_means_a_loud_failure():
 # --------------------------------------------------------------------------
 # the compiled kernels
 # --------------------------------------------------------------------------
+def test_a_library_older_than_the_sources_is_never_used(tmp_path, monkeypatch):
+    import importlib
+
+    build = importlib.import_module("fms_amd.kernels.build")
+    folder = tmp_path / "built"
+    folder.mkdir()
+    lib = folder / build.LIB_NAME
+    lib.write_bytes(b"not a library; only its digest is looked at")
+    monkeypatch.setattr(build, "build_dirs", lambda: [str(folder)])
+    calls = []
+
+    def fake_build(verbose=True):
+        calls.append("build")
+        return "rebuilt"
+
+    monkeypatch.setattr(build, "build", fake_build)
+    (folder / build.DIGEST_NAME).write_text(build.source_digest())
+    assert build.ensure_built(verbose=False) == str(lib) and calls == []
+    (folder / build.DIGEST_NAME).write_text("0" * 64)  # built from other sources
+    assert build.ensure_built(verbose=False) == "rebuilt" and calls == ["build"]
+    (folder / build.DIGEST_NAME).unlink()  # no record of what it was built from
+    assert build.ensure_built(verbose=False) == "rebuilt"
+
+    def no_compiler(verbose=True):
+        raise RuntimeError("hipcc was not found")
+
+    monkeypatch.setattr(build, "build", no_compiler)
+    with pytest.raises(RuntimeError, match="does not match the present sources"):
+        build.ensure_built(verbose=False)
+
+
 def test_kernels_compile_without_relative_register_indexing(tmp_path):
     """A private array indexed by a run-time value is addressed through relative register
     indexing (s_set_gpr_idx / v_movrel); the compiler may then write the indexed register
