@@ -74,9 +74,11 @@ class DecodeGraph:
         self.n_pages: List[int] = []
         self.stamps: List[int] = []  # the cache's stamp of every sequence after the last replay
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
 
     def _run(self) -> None:
         logits = self.engine.model.forward(self.batch, self.engine.cache)
+        self.logits = logits  # [rows, vocab]; after a replay, that step's logits (padding rows: anything)
         s = self.sampling
         ops.sample(logits, s.do_sample, s.temperature, s.top_k or 0, self.rng if s.do_sample else None, out=self.tokens)
         ops.advance_positions_(self.positions, self.seq_of_token)

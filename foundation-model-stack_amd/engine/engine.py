@@ -44,6 +44,7 @@ class Engine:
         self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", True) for p in model.walk())
         self._graphs = {}
         self.graph_captures = []  # (rows, context bound) of every capture, in order
+        self.last_graph: Optional[DecodeGraph] = None  # the graph of the last replayed step (its .logits are that step's)
 
     # ---- sequences ---------------------------------------------------------
     def new_sequence(self) -> int:
@@ -114,6 +115,7 @@ class Engine:
         else:
             graph.load(slots, tokens, positions, seeds or [0] * len(slots), counters or [0] * len(slots))
         graph.stamps = [self.cache.stamp(s) for s in slots]
+        self.last_graph = graph
         return graph.replay()
 
     def prepare(self, slots, tokens, want) -> StepBatch:

@@ -165,13 +165,28 @@ def gated_feed_forward(
     bias_fused: Optional[torch.Tensor] = None,
     bias2: Optional[torch.Tensor] = None,
     storage=None,
+    rounding: str = "stored",
 ) -> torch.Tensor:
-    """fms/modules/feedforward.py:288-297: first half of the fused rows is the gate."""
+    """fms/modules/feedforward.py:288-297: first half of the fused rows is the gate.
+
+    rounding "reference": the activation and the product are two operations of the model dtype there
+    (self.a(out1) * out2), so each of them rounds."""
     st = _stored(storage)
     hidden = wg1_fused.shape[0] // 2
     both = st(linear(x, wg1_fused, bias_fused))
     gate, up = both[..., :hidden], both[..., hidden:]
-    return linear(st(silu(gate) * up), w2, bias2)
+    act = st(silu(gate)) if rounding == "reference" else silu(gate)
+    return linear(st(act * up), w2, bias2)
+
+
+def rms_norm_as_stored(x: torch.Tensor, weight: torch.Tensor, eps: float, storage) -> torch.Tensor:
+    """fms/modules/layernorm.py:60-66 in a model dtype below float32: the statistics and the scaling are
+    float32, the scaled row is cast to the model dtype (`.type_as(x)`), and only then multiplied by the
+    weight, in the model dtype: two roundings."""
+    st = _stored(storage)
+    xf = x.float()
+    xf = st(xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps))
+    return st(st(weight.float()) * xf)
 
 
 def _stored(storage):
@@ -205,21 +220,48 @@ def attention_block(
     return st(linear(mixed.reshape(S, H * D), dense_w, dense_b))
 
 
+def rotated_queries_and_keys(weights: Dict[str, torch.Tensor], cfg: PlainConfig, ids: List[int], layer: int = 0):
+    """Queries [S, H, D] and keys [S, K, D] of the first layer after the rotation (tests use them to see how
+    sharp a model's attention is); only layer 0 can be had without running the layers before it."""
+    if layer != 0:
+        raise ValueError("only the first layer's queries and keys depend on nothing but the embedding")
+    w = {name: t.float() for name, t in weights.items()}
+    S, H, K, D = len(ids), cfg.nheads, cfg.kvheads, cfg.head_dim
+    p = "base_model.layers.0."
+    x = embedding(w["base_model.embedding.weight"], torch.as_tensor(ids, dtype=torch.long))
+    h = rms_norm(x, w[p + "ln.weight"], cfg.eps)
+    qkv = linear(h, w[p + "attn.in_proj.qkv_fused.weight"], w.get(p + "attn.in_proj.qkv_fused.bias"))
+    q, k, _ = torch.split(qkv, [H * D, K * D, K * D], dim=-1)
+    freqs = rope_frequencies(D, cfg.theta, cfg.rope_scaling)
+    positions = torch.arange(S)
+    return rope_rotate(q.reshape(S, H, D), positions, freqs), rope_rotate(k.reshape(S, K, D), positions, freqs)
+
+
 def forward(
     weights: Dict[str, torch.Tensor],
     cfg: PlainConfig,
     ids: List[int],
     first_position: int = 0,
     storage=None,
+    rounding: str = "stored",
 ) -> torch.Tensor:
     """fms/models/llama.py:137-162, 332-353, 444-445: logits [S, V] of one whole sequence.
 
-    storage=torch.bfloat16 rounds every tensor that the reference would hold in its model dtype
-    (the outputs of norms, linears, rotation, attention and the gate product) and computes the
-    rest in float32 as the reference does (norm statistics, rotation).  It serves to size the
-    error that bfloat16 storage alone causes; the residual stream and the logits stay float32.
+    storage=torch.bfloat16 sizes the error of running in bfloat16; `rounding` says where it rounds.
+    "stored": every tensor that is stored between two operations (the outputs of norms, linears, rotation,
+    attention and the gate product) is rounded once; the residual stream, the norm's multiplication by its
+    weight and the logits stay float32.  "reference": the roundings of the reference run in that dtype:
+    besides the above, the norm rounds before and after its weight (layernorm.py:60-66), the residual sums
+    are sums of the model dtype (llama.py:153, 162), the embedding row and the activation round, and the
+    logits leave the head in the model dtype (llama.py:445).  Norm statistics and the rotation are float32
+    in both, as in the reference.
     """
+    if rounding not in ("stored", "reference"):
+        raise ValueError(rounding)
     st = _stored(storage)
+    ref = rounding == "reference"
+    rs = st if ref else (lambda t: t)  # roundings that only the reference's arithmetic has
+    norm = (lambda x, w_: rms_norm_as_stored(x, w_, cfg.eps, storage)) if ref else (lambda x, w_: st(rms_norm(x, w_, cfg.eps)))
     w = {name: t.float() for name, t in weights.items()}
     tokens = torch.as_tensor(ids, dtype=torch.long)
     positions = torch.arange(len(ids)) + first_position
@@ -227,11 +269,11 @@ def forward(
         # tests/modules/test_positions.py:156-168: a position beyond the table raises
         raise IndexError("position beyond max_expected_seq_len")
     freqs = rope_frequencies(cfg.head_dim, cfg.theta, cfg.rope_scaling)
-    x = embedding(w["base_model.embedding.weight"], tokens)
+    x = rs(embedding(w["base_model.embedding.weight"], tokens))
     for i in range(cfg.nlayers):
         p = f"base_model.layers.{i}."
         residual = x
-        h = st(rms_norm(x, w[p + "ln.weight"], cfg.eps))
+        h = norm(x, w[p + "ln.weight"])
         h = attention_block(
             h,
             positions,
@@ -243,9 +285,9 @@ def forward(
             w.get(p + "attn.dense.bias"),
             storage,
         )
-        x = h + residual
+        x = rs(h + residual)
         residual = x
-        h = st(rms_norm(x, w[p + "ff_ln.weight"], cfg.eps))
+        h = norm(x, w[p + "ff_ln.weight"])
         h = st(gated_feed_forward(
             h,
             w[p + "ff_sub_layer.wg1_fused.weight"],
@@ -253,11 +295,12 @@ def forward(
             w.get(p + "ff_sub_layer.wg1_fused.bias"),
             w.get(p + "ff_sub_layer.w2.bias"),
             storage,
+            rounding,
         ))
-        x = h + residual
-    x = st(rms_norm(x, w["base_model.dec_norm.weight"], cfg.eps))
+        x = rs(h + residual)
+    x = norm(x, w["base_model.dec_norm.weight"])
     head = w["base_model.embedding.weight"] if cfg.tie_heads and "head.weight" not in w else w["head.weight"]
-    return linear(x, head)
+    return rs(linear(x, head))
 
 
 # ----------------------------------------------------------------------------

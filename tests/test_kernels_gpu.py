@@ -356,6 +356,33 @@ def test_gemm_bf16(ops, M, N, K):
     torch.testing.assert_close(out.double(), want, atol=3e-2, rtol=1e-2)
 
 
+@pytest.mark.parametrize("M", [1, 5, 17, 64, 70, 200])
+@pytest.mark.parametrize("N,K", [(37, 12), (100, 44), (60, 50), (301, 1000 + 4)])
+def test_gemm_bf16_of_widths_that_are_no_multiple_of_8(ops, M, N, K):
+    """Rows of such widths are not 16-byte aligned, which the MFMA kernels need: an element-wise kernel takes
+    them, so that no width a configuration allows is refused.  Also a view whose row stride is odd."""
+    torch.manual_seed(17)
+    x = torch.randn(M, K).to(torch.bfloat16)
+    w = (torch.randn(N, K) * 0.1).to(torch.bfloat16)
+    b = torch.randn(N).to(torch.bfloat16)
+    want = x.double() @ w.double().t()
+    for out_dtype in (torch.bfloat16, torch.float32):
+        out = ops.linear(dev(x), dev(w), None, out_dtype=out_dtype).cpu()
+        assert out.dtype == out_dtype
+        torch.testing.assert_close(out.double(), want, atol=3e-2 if out_dtype == torch.bfloat16 else 2e-3, rtol=1e-2)
+    for bias in (b, b.float()):
+        out = ops.linear(dev(x), dev(w), dev(bias), out_dtype=torch.float32).cpu()
+        torch.testing.assert_close(out.double(), want + b.double(), atol=2e-3, rtol=1e-2)
+    wide = dev(torch.randn(M, K + 3).to(torch.bfloat16))
+    out = ops.linear(wide[:, :K], dev(w), None, out_dtype=torch.float32).cpu()
+    torch.testing.assert_close(out.double(), wide[:, :K].cpu().double() @ w.double().t(), atol=2e-3, rtol=1e-2)
+    if N % 2 == 0:
+        out = ops.gated_linear(dev(x), dev(w), dev(b), "swish").cpu().float()
+        gu = x.float() @ w.float().t() + b.float()
+        want = P.silu(gu[:, : N // 2]) * gu[:, N // 2 :]
+        torch.testing.assert_close(out, want, atol=4e-2, rtol=2e-2)
+
+
 @pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100])
 @pytest.mark.parametrize("hidden,K", [(44, 24), (77, 40), (176, 64), (1000, 96)])
 def test_gated_linear(ops, M, hidden, K):
@@ -497,8 +524,9 @@ def test_sampling_ties_at_threshold_survive(ops):
 def test_kernels_refuse_what_they_cannot_do(ops):
     from fms_amd.kernels import KernelError
 
-    with pytest.raises((KernelError, ValueError)):
-        ops.linear(dev(torch.zeros(2, 12, dtype=torch.bfloat16)), dev(torch.zeros(8, 12, dtype=torch.bfloat16)))  # K % 8
+    with pytest.raises((KernelError, ValueError)):  # a deferred row norm needs rows the MFMA kernels can load
+        ops.linear(dev(torch.zeros(2, 12, dtype=torch.bfloat16)), dev(torch.zeros(8, 12, dtype=torch.bfloat16)),
+                   row_norm=ops.RowNorm(dev(torch.zeros(2, 1)), 1e-5))
     with pytest.raises(RuntimeError):
         ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4))  # CPU tensors: no CPU path
     with pytest.raises((KernelError, ValueError)):

@@ -1,0 +1,190 @@
+"""The engine at the layer sizes that are served and measured: two layers of the Llama-3-8B shape (grouped kv
+heads) and of the Llama-2-7B shape (as many kv heads as heads), with a vocabulary cut to 4096 so that the plain
+implementation on the CPU stays cheap.  These sizes take other kernels than the tiny configurations do: the
+prefill attention with its head size known at compile time, the decode attention that stages pages in LDS, the
+weight-streaming products with thousands of columns and their variants for 17 to 64 rows, vendor products above
+64 rows.  float32 and bfloat16 against the plain implementation, and bfloat16 against the engine's own float32
+path: whole prompts, the last 32 tokens one by one, ragged batches with reused slots, and decode batches of 5,
+24, 64 and 80 sequences through captured graphs.
+
+The cache-consistency check of the reference's benchmark script (scripts/benchmark_inference.py:197-213: a cached
+one-token step against the full recomputation) and its heterogeneous-batch test (tests/utils/test_generate.py:
+77-136) are the nearest things it has."""
+
+import gc
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+import plain_llama as P  # noqa: E402
+from gpu_checks import MARGIN, check, expect  # noqa: E402
+
+SHAPES = {
+    "llama3_8b_layers": dict(src_vocab_size=4096, emb_dim=4096, nheads=32, kvheads=8, nlayers=2, hidden_dim=14336,
+                             multiple_of=1, norm_eps=1e-5, rope_theta=500000.0, max_expected_seq_len=4096),
+    "llama2_7b_layers": dict(src_vocab_size=4096, emb_dim=4096, nheads=32, kvheads=0, nlayers=2, hidden_dim=11008,
+                             multiple_of=1, norm_eps=1e-5, rope_theta=10000.0, max_expected_seq_len=4096),
+}
+DTYPES = ["float32", "bfloat16"]
+
+
+class Shape:
+    def __init__(self, name, folder, lib):
+        self.name, self.folder, self.lib = name, folder, lib
+        self.cfg, self.weights = P.load_model_folder(folder)
+        self.models = {}
+
+    def model(self, dtype):
+        if dtype not in self.models:
+            self.models[dtype] = self.lib.get_model("hf_pretrained", model_path=self.folder, data_type=dtype)
+        return self.models[dtype]
+
+    def tokens(self, n, seed):
+        g = torch.Generator().manual_seed(seed)
+        return torch.randint(0, self.cfg.vocab, (n,), generator=g).tolist()
+
+
+@pytest.fixture(scope="module", params=sorted(SHAPES))
+def shape(request, tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import fms_amd
+    from fms_amd.kernels import load
+
+    load()
+    folder = str(tmp_path_factory.mktemp(request.param))
+    # the weights of the benchmark (N(0, 0.02)), and norm scales that are not all one, so that a norm in the wrong place shows
+    fms_amd.write_model_folder(folder, fms_amd.LLaMAConfig(**SHAPES[request.param]), seed=17, std=0.02, norm_std=0.1)
+    print(f"[{request.param}] model folder written", flush=True)
+    s = Shape(request.param, folder, fms_amd)
+    yield s
+    s.models.clear()
+    del s
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_whole_prompt_and_last_32_tokens_one_by_one(shape, dtype):
+    from fms_amd.engine import Engine
+
+    engine = Engine(shape.model(dtype), max_tokens=1024, max_slots=1)
+    ids = shape.tokens(700, 1)
+    want = expect(shape.weights, shape.cfg, ids, dtype)
+    slot = engine.new_sequence()
+    check(engine.step([slot], [ids], "all"), want, dtype)
+    engine.end_sequence(slot)
+    slot = engine.new_sequence()
+    got = [engine.step([slot], [ids[:-32]], "all")]
+    for tok in ids[-32:]:
+        got.append(engine.step([slot], [[tok]], "last"))
+    engine.end_sequence(slot)
+    check(torch.cat(got), want, dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_ragged_batches_with_early_ends_and_reused_slots(shape, dtype):
+    from fms_amd.engine import Engine
+
+    engine = Engine(shape.model(dtype), max_tokens=12 * 64, max_slots=5)  # the first round fills every page
+    rounds = [
+        [(70, 3), (5, 9), (200, 2), (129, 1), (64, 6)],  # (prompt length, decoded tokens)
+        [(33, 8), (300, 4), (1, 5)],
+    ]
+    seed = 100
+    for requests in rounds:
+        seqs = []
+        for prompt_len, n_decode in requests:
+            seed += 1
+            seqs.append(dict(ids=shape.tokens(prompt_len + n_decode, seed), prompt=prompt_len, slot=engine.new_sequence(),
+                             got=[], at=prompt_len))
+        logits = engine.step([s["slot"] for s in seqs], [s["ids"][: s["prompt"]] for s in seqs], "all")
+        row = 0
+        for s in seqs:
+            s["got"].append(logits[row : row + s["prompt"]])
+            row += s["prompt"]
+        alive = list(seqs)
+        while alive:
+            for s in alive:
+                if s["at"] == len(s["ids"]):
+                    engine.end_sequence(s["slot"])  # ends earlier: its slot and pages go back while the others go on
+            alive = [s for s in alive if s["at"] < len(s["ids"])]
+            if not alive:
+                break
+            logits = engine.step([s["slot"] for s in alive], [[s["ids"][s["at"]]] for s in alive], "last")
+            for i, s in enumerate(alive):
+                s["got"].append(logits[i : i + 1])
+                s["at"] += 1
+        engine.cache.check()
+        assert engine.cache.live_slots() == []
+        for s in seqs:
+            check(torch.cat(s["got"]), expect(shape.weights, shape.cfg, s["ids"], dtype), dtype)
+
+
+def prompt_lengths(n):
+    special = [63, 64, 65, 1, 127, 128, 191, 320]
+    return [(special[i] if i < len(special) else 2 + (53 * i * i + 17 * i) % 250) for i in range(n)]
+
+
+@pytest.mark.parametrize("n_seqs", [5, 24, 64, 80])
+def test_decode_batches_through_graphs(shape, n_seqs):
+    """bfloat16 decode steps of 5, 24, 64 and 80 sequences of unequal lengths, as generation runs them
+    (decode_and_choose: a captured graph, the token choice inside it), against the engine's float32 path fed
+    the same tokens, and both against the plain implementation.  After three steps every third sequence ends."""
+    from fms_amd.engine import Engine
+    from fms_amd.sampling import SamplingParams
+
+    greedy = SamplingParams(do_sample=False)
+    lens = prompt_lengths(n_seqs)
+    room = sum(-(-(n + 8) // 64) * 64 for n in lens)
+    half = Engine(shape.model("bfloat16"), max_tokens=room, max_slots=n_seqs, use_graphs=True)
+    full = Engine(shape.model("float32"), max_tokens=room, max_slots=n_seqs, use_graphs=False)
+    assert half.use_graphs
+    seqs = [dict(ids=shape.tokens(n, 700 + 3 * n_seqs + i), n=n, half=[], full=[]) for i, n in enumerate(lens)]
+    for engine, key in ((half, "slot_h"), (full, "slot_f")):
+        for s in seqs:
+            s[key] = engine.new_sequence()
+        for i in range(0, n_seqs, 16):
+            group = seqs[i : i + 16]
+            logits = engine.step([s[key] for s in group], [s["ids"] for s in group], "last")
+            if engine is full:
+                for s, tok in zip(group, logits.argmax(-1).tolist()):
+                    s["next"] = tok
+    alive = list(seqs)
+    for step in range(6):
+        if step == 3:
+            for s in alive[::3]:
+                half.end_sequence(s["slot_h"])
+                full.end_sequence(s["slot_f"])
+            alive = [s for i, s in enumerate(alive) if i % 3]
+        fed = [s["next"] for s in alive]
+        chosen = half.decode_and_choose([s["slot_h"] for s in alive], fed, greedy)
+        from_graph = half.last_graph.logits[: len(alive)].float().cpu()
+        assert chosen == from_graph.argmax(-1).tolist()
+        exact = full.step([s["slot_f"] for s in alive], [[t] for t in fed], "last").cpu()
+        for s, tok, row_h, row_f in zip(alive, chosen, from_graph, exact):
+            s["ids"] = s["ids"] + [s["next"]]
+            s["half"].append(row_h)
+            s["full"].append(row_f)
+            s["next"] = tok
+    for s in alive:
+        half.end_sequence(s["slot_h"])
+        full.end_sequence(s["slot_f"])
+    half.cache.check()
+    assert half.cache.live_slots() == [] == full.cache.live_slots()
+    assert len(half.graph_captures) >= 2  # the batch before and after the early ends
+    # against the plain implementation: the sequences around the page borders and every eighth of the others
+    largest = 0.0
+    for i, s in enumerate(seqs):
+        if i < 8 or i % 8 == 0:
+            want = expect(shape.weights, shape.cfg, s["ids"], "bfloat16")[s["n"] :]
+            check(torch.stack(s["half"]), want, "bfloat16")
+            check(torch.stack(s["full"]), want.logits, "float32")
+            largest = max(largest, float(want.ref_error.max()))
+    # every sequence: the bfloat16 graph against the float32 path (which the check above ties to the plain
+    # implementation), no further apart than the reference's own bfloat16 error on the sequences above
+    for i, s in enumerate(seqs):
+        error = float((torch.stack(s["half"]) - torch.stack(s["full"])).abs().max())
+        assert error <= MARGIN * largest, f"sequence {i} ({s['n']} prompt tokens): bfloat16 is {error:.4g} from float32"

@@ -246,6 +246,34 @@ def test_forward_prefix_property():
         P.forward(weights, cfg, list(range(40)), first_position=30)
 
 
+def test_bfloat16_roundings_of_the_reference():
+    """fms/modules/layernorm.py:60-66 in bfloat16 is the module's own sequence of casts; and a model run with
+    the reference's roundings differs from the float32 one by bfloat16-sized errors, a little more than a run
+    that rounds stored tensors only (it rounds in more places)."""
+    torch.manual_seed(4)
+    x = (torch.randn(7, 48) * 3).bfloat16()
+    w = (1 + 0.3 * torch.randn(48)).bfloat16()
+    xf = x.float()
+    want = w * (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + 1e-5)).type_as(x)  # bfloat16 * bfloat16
+    assert want.dtype == torch.bfloat16
+    got = P.rms_norm_as_stored(x.float(), w.float(), 1e-5, torch.bfloat16)
+    assert torch.equal(got, want.float())
+    assert not torch.equal(got, P.rms_norm(x.float(), w.float(), 1e-5).bfloat16().float())  # one rounding is not two
+
+    cfg = P.PlainConfig(vocab=50, width=32, nheads=4, kvheads=2, nlayers=3, hidden=72, eps=1e-5, theta=1e4, max_len=64)
+    weights = {k: (v * 3).bfloat16().float() for k, v in _fixture_weights(cfg, 12).items()}
+    ids = list(range(5, 45))
+    exact = P.forward(weights, cfg, ids)
+    stored = P.forward(weights, cfg, ids, storage=torch.bfloat16)
+    reference = P.forward(weights, cfg, ids, storage=torch.bfloat16, rounding="reference")
+    assert torch.equal(reference, reference.bfloat16().float())  # the reference's logits are bfloat16 numbers
+    scale = float(exact.abs().max())
+    e_stored, e_ref = float((stored - exact).abs().max()), float((reference - exact).abs().max())
+    assert 1e-4 * scale < e_stored < 0.05 * scale and 1e-4 * scale < e_ref < 0.05 * scale
+    assert float((stored - exact).abs().mean()) < float((reference - exact).abs().mean())
+    assert torch.equal(P.forward(weights, cfg, ids, storage=torch.float32, rounding="reference"), exact)
+
+
 def test_sampling_distribution():
     logits = torch.tensor([1.0, 3.0, 2.0, 3.0, -1.0])
     p = P.sampling_distribution(logits, 0.5, 2)
