@@ -140,6 +140,17 @@ long fmsamd_argmax_workspace(int rows, int vocab);
 int fmsamd_argmax(const float* logits, long ld, int rows, int vocab, void* workspace, long workspace_bytes,
                   int* out_tokens, hipStream_t stream);
 
+// The greedy choice of fmsamd_argmax without a workspace, for callers that cannot allocate device memory:
+// code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart
+// in the reference.  The partial results of the first stage go to an array of FMSAMD_ARGMAX_STATIC_BYTES
+// that the library holds on every GPU it runs on until the process ends; rows * ceil(vocab / 2048) * 8 bytes
+// must fit (32768 partial results: 256 rows of a vocabulary of 262144, 1024 rows of one of 65536), larger
+// inputs are refused.  The call allocates nothing and frees nothing.  All calls on one GPU share that GPU's
+// array: calls that overlap in time on one GPU (two streams, two threads) race; calls on one stream do not.
+// The first call on a device looks the array's address up (hipGetSymbolAddress), so make it outside a capture.
+#define FMSAMD_ARGMAX_STATIC_BYTES (256 * 1024)
+int fmsamd_argmax_static(const float* logits, long ld, int rows, int vocab, int* out_tokens, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

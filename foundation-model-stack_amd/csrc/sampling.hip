@@ -5,6 +5,8 @@
 //               a uniform number drawn from a counter-based generator.
 // The generator state of a row is (seed, counter) in device memory; the
 // kernel advances the counter, so that a captured graph can be replayed.
+#include <mutex>
+
 #include "common.h"
 #include "fmsamd.h"
 
@@ -219,6 +221,58 @@ extern "C" int fmsamd_argmax(const float* logits, long ld, int rows, int vocab, 
   FMS_LAUNCH_CHECK("argmax_partial");
   argmax_final_kernel<<<rows, ARG_THREADS, 0, stream>>>(part_val, part_idx, chunks, out_tokens);
   FMS_LAUNCH_CHECK("argmax_final");
+  return 0;
+}
+
+// ---- the same greedy choice for callers that cannot allocate ---------------------------------
+// The partial maxima of the first stage live in an array of the library's own instead of a workspace of the
+// caller's.  In host code the array's name is only a handle: its address on the current GPU is asked for
+// once per device (every GPU holds a copy of its own) and that address is what the kernels get.
+static __device__ __align__(256) unsigned char scratch[FMSAMD_ARGMAX_STATIC_BYTES];
+
+#define ARG_MAX_DEVICES 64
+static void* scratch_of_device[ARG_MAX_DEVICES];
+static std::mutex scratch_lock;
+
+static int scratch_address(void** out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  FMS_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  FMS_REQUIRE(device >= 0 && device < ARG_MAX_DEVICES, "argmax_static: device %d is beyond the %d this library keeps track of",
+              device, ARG_MAX_DEVICES);
+  std::lock_guard<std::mutex> guard(scratch_lock);
+  if (scratch_of_device[device] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    FMS_REQUIRE(e == hipSuccess && ptr != nullptr, "argmax_static: the scratch array has no address on device %d: %s", device,
+                hipGetErrorString(e));
+    scratch_of_device[device] = ptr;
+  }
+  *out = scratch_of_device[device];
+  return 0;
+}
+
+extern "C" int fmsamd_argmax_static(const float* logits, long ld, int rows, int vocab, int* out_tokens,
+                                    hipStream_t stream) {
+  if (rows == 0) return 0;
+  FMS_REQUIRE(rows > 0 && vocab > 0 && ld >= vocab, "argmax_static: bad sizes rows=%d vocab=%d ld=%ld", rows, vocab, ld);
+  FMS_REQUIRE(rows <= 65535, "argmax_static: %d rows exceed one launch", rows);
+  FMS_REQUIRE(logits != nullptr && out_tokens != nullptr, "argmax_static: null logits or output");
+  const int chunks = ceil_div(vocab, ARG_CHUNK);
+  const long need = fmsamd_argmax_workspace(rows, vocab);
+  FMS_REQUIRE(need <= (long)FMSAMD_ARGMAX_STATIC_BYTES,
+              "argmax_static: %d rows of %d logits need %ld bytes of partial results, the library's array holds %ld "
+              "(rows x ceil(vocab / %d) <= %ld): use fmsamd_argmax with a workspace",
+              rows, vocab, need, (long)FMSAMD_ARGMAX_STATIC_BYTES, ARG_CHUNK, (long)FMSAMD_ARGMAX_STATIC_BYTES / 8);
+  void* base = nullptr;
+  if (scratch_address(&base) != 0) return -1;
+  // every entry that the second stage reads is written by the first: nothing has to start at zero
+  float* part_val = (float*)base;
+  int* part_idx = (int*)(part_val + (size_t)rows * chunks);
+  argmax_partial_kernel<<<dim3(chunks, rows), ARG_THREADS, 0, stream>>>(logits, ld, vocab, part_val, part_idx, chunks);
+  FMS_LAUNCH_CHECK("argmax_static (first stage)");
+  argmax_final_kernel<<<rows, ARG_THREADS, 0, stream>>>(part_val, part_idx, chunks, out_tokens);
+  FMS_LAUNCH_CHECK("argmax_static (second stage)");
   return 0;
 }
 
