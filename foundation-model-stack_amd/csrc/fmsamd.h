@@ -113,9 +113,9 @@ int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const 
                                   const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
                                   hipStream_t stream);
 // resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, partial_count] = sums
-// of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(M, N) says;
+// of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(M, N, K) says;
 // every entry is written).  At most 64 rows.
-int fmsamd_gemm_skinny_residual_partials(int M, int N);
+int fmsamd_gemm_skinny_residual_partials(int M, int N, int K);
 int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                      float* resid, long ldr, const void* norm_w, int norm_w_dtype, void* scaled,
                                      long ldo, float* partials, int partial_count, int M, int N, int K,

@@ -223,7 +223,8 @@ extern "C" int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const vo
 // UNR: groups of 128 k-values whose loads a wave issues before it multiplies: what keeps enough
 // bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 4 loads of 16 bytes outstanding).
 template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typename BiasT>
-__global__ void __launch_bounds__(SK_WAVES* WAVE) __attribute__((amdgpu_waves_per_eu(4)))  // two blocks a compute unit
+__global__ void __launch_bounds__(SK_WAVES* WAVE)
+    __attribute__((amdgpu_waves_per_eu(MT > 1 ? 2 : 4)))  // two blocks a compute unit; one with several tiles of x
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
                        int rows_per_block, RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
@@ -547,7 +548,13 @@ static void launch_skinny(const void* x, long ldx, const void* w, const void* bi
 // of 14336 columns in blocks of 14 gate rows and 14 up rows is four blocks a unit of 28 rows where blocks of 16
 // and 16 are three and a half - that is, four for some - of 32.
 #define SK_COMPUTE_UNITS 256
-static int skinny_x_rows(int M) { return ceil_div(M < 16 ? M : 16, 4) * 4; }
+static int skinny_x_rows(int M) { return ceil_div(M, 4) * 4; }
+
+// 17 to 32 rows of x and a short K: the kernel above with two tiles of x a wave beats the kernels of
+// gemm_wide.hip, which have to cut so short a K into slices that meet in memory and need a second kernel
+// (measured at K = 4096: 13.5 against 17.2 us for 6144 weight rows, 11.3 against 14.5 for 4096; at K = 14336, and
+// from 33 rows on, where every block reads more of x than of W, the wide kernels win).
+static bool skinny_takes_many_rows(int M, int N, int K) { return M > 16 && M <= 32 && K <= 8192; }
 
 static int skinny_rows_per_block(int N, int M) {
   int best = 0;
@@ -591,16 +598,24 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N, "gemm_skinny_bf16: leading dimensions too small");
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_bf16: unknown output dtype %d", out_dtype);
-  if (M > 16)
+  if (M > 16 && !skinny_takes_many_rows(M, N, K))
     return wide_product(EPI_PLAIN, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, scale, RopeEpilogue{},
                         ResidEpilogue{}, workspace, workspace_bytes, stream);
   const int rows = skinny_rows_per_block(N, M);
 #define FMS_LS(NTB, MT) \
   launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, rows, stream, scale)
+#define FMS_LS_MT(NTB)  \
+  do {                  \
+    if (M <= 16)        \
+      FMS_LS(NTB, 1);   \
+    else                \
+      FMS_LS(NTB, 2);   \
+  } while (0)
   if (rows > 16)
-    FMS_LS(2, 1);
+    FMS_LS_MT(2);
   else
-    FMS_LS(1, 1);
+    FMS_LS_MT(1);
+#undef FMS_LS_MT
 #undef FMS_LS
   FMS_LAUNCH_CHECK("gemm_skinny_bf16");
   return 0;
@@ -659,16 +674,24 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   FMS_REQUIRE(cos_t == nullptr || (max_pos > 0 && sin_t != nullptr), "qkv_rope_skinny_bf16: empty rotary table");
   RopeEpilogue rope{positions, seq_of_token, block_table, table_stride, rot_dim > 0 ? cos_t : nullptr, sin_t, rot_dim,
                     max_pos, (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim};
-  if (M > 16)
+  if (M > 16 && !skinny_takes_many_rows(M, N, K))
     return wide_product(EPI_ROPE, x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, scale, rope,
                         ResidEpilogue{}, workspace, workspace_bytes, stream);
   const int rows = skinny_rows_per_block(N, M);
 #define FMS_LR(NTB, MT) \
   launch_skinny<NTB, MT, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
+#define FMS_LR_MT(NTB)  \
+  do {                  \
+    if (M <= 16)        \
+      FMS_LR(NTB, 1);   \
+    else                \
+      FMS_LR(NTB, 2);   \
+  } while (0)
   if (rows > 16)
-    FMS_LR(2, 1);
+    FMS_LR_MT(2);
   else
-    FMS_LR(1, 1);
+    FMS_LR_MT(1);
+#undef FMS_LR_MT
 #undef FMS_LR
   FMS_LAUNCH_CHECK("qkv_rope_skinny_bf16");
   return 0;
@@ -679,18 +702,18 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
 //   scaled[M, N] = resid * norm_w                      bfloat16: the next norm's input, not yet divided by its
 //                                                      root mean square
 //   partials[m, i] = sums of resid[m]^2 over groups of up to 16 columns, the unused ones zero
-//                    [M, partial_count], partial_count >= fmsamd_gemm_skinny_residual_partials(N)
+//                    [M, partial_count], partial_count >= fmsamd_gemm_skinny_residual_partials(M, N, K)
 // A product that takes `scaled` with these partials as its deferred row norm then equals the product of the
 // normed stream.  M <= 64.
-extern "C" int fmsamd_gemm_skinny_residual_partials(int M, int N) {
-  if (M > 16) return ceil_div(N, 16);
+extern "C" int fmsamd_gemm_skinny_residual_partials(int M, int N, int K) {
+  if (M > 16 && !skinny_takes_many_rows(M, N, K)) return ceil_div(N, 16);
   const int rows = skinny_rows_per_block(N, M);
   return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
 }
 
 // Bytes of workspace that the products for at most 64 rows need (none up to 16 rows).  rows: all rows of W.
 extern "C" long fmsamd_gemm_skinny_workspace(int M, int rows, int K) {
-  return M > 16 && M <= 64 ? wide_workspace_bytes(M, rows, K) : 0;
+  return M > 16 && M <= 64 ? wide_workspace_bytes(M, rows, K) : 0;  // enough for every product of this shape
 }
 
 extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias,
@@ -710,11 +733,11 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
   const int rows = skinny_rows_per_block(N, M);
-  const int tiles = fmsamd_gemm_skinny_residual_partials(M, N);
+  const int tiles = fmsamd_gemm_skinny_residual_partials(M, N, K);
   FMS_REQUIRE(partial_count >= tiles, "gemm_skinny_residual_bf16: room for %d partial sums per row, %d needed",
               partial_count, tiles);
   ResidEpilogue res{resid, ldr, norm_w, norm_w_dtype == FMS_F32, partials, partial_count};
-  if (M > 16) {
+  if (M > 16 && !skinny_takes_many_rows(M, N, K)) {
     res.tiles = tiles;  // the finish kernel writes exactly these
     FMS_REQUIRE(partial_count == tiles, "gemm_skinny_residual_bf16: %d partial sums per row, %d expected", partial_count,
                 tiles);
@@ -724,10 +747,18 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
 #define FMS_LX(NTB, MT)                                                                                              \
   launch_skinny<NTB, MT, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, \
                                     scale, RopeEpilogue{}, res)
+#define FMS_LX_MT(NTB)  \
+  do {                  \
+    if (M <= 16)        \
+      FMS_LX(NTB, 1);   \
+    else                \
+      FMS_LX(NTB, 2);   \
+  } while (0)
   if (rows > 16)
-    FMS_LX(2, 1);
+    FMS_LX_MT(2);
   else
-    FMS_LX(1, 1);
+    FMS_LX_MT(1);
+#undef FMS_LX_MT
 #undef FMS_LX
   FMS_LAUNCH_CHECK("gemm_skinny_residual_bf16");
   return 0;

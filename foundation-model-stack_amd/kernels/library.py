@@ -43,7 +43,7 @@ _SIGNATURES = {
     "fmsamd_gemm_skinny_workspace": [I, I, I],
     "fmsamd_gemm_skinny_bf16": [P, L, P, P, I, P, I, L, I, I, I, P, P, L, P],
     "fmsamd_gemm_skinny_gated_bf16": [P, L, P, P, I, P, I, L, I, I, I, I, P, P, L, P],
-    "fmsamd_gemm_skinny_residual_partials": [I, I],
+    "fmsamd_gemm_skinny_residual_partials": [I, I, I],
     "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P, L, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],

@@ -527,7 +527,7 @@ def linear_into_stream(
         raise ValueError(f"the norm weight is a contiguous float32 or bfloat16 [{N}] tensor")
     scaled = torch.empty(M, N, dtype=torch.bfloat16, device=x.device)
     lib = load()
-    partials = torch.empty(M, lib.fmsamd_gemm_skinny_residual_partials(M, N), dtype=torch.float32, device=x.device)
+    partials = torch.empty(M, lib.fmsamd_gemm_skinny_residual_partials(M, N, K), dtype=torch.float32, device=x.device)
     ws, ws_bytes = _skinny_workspace(M, N, K, x.device)
     check(lib.fmsamd_gemm_skinny_residual_bf16(
         x.data_ptr(), x.stride(0), weight.data_ptr(), _ptr(bias), _code(bias.dtype) if bias is not None else 0,
