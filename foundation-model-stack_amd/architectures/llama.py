@@ -51,7 +51,7 @@ def llama_spec(config: LLaMAConfig) -> ModelSpec:
     return ModelSpec(
         vocab=config.src_vocab_size,
         width=config.emb_dim,
-        max_seq_len=config.max_expected_seq_len,
+        max_seq_len=config.max_positions,
         layers=[layer for _ in range(config.nlayers)],
         final_norm=norm,
         positions={
@@ -61,6 +61,7 @@ def llama_spec(config: LLaMAConfig) -> ModelSpec:
                     "dim": config.head_dim,
                     "theta": config.rope_theta,
                     "max_seq_len": config.max_expected_seq_len,
+                    "max_positions": config.max_positions,
                     "scaling": dict(config.rope_scaling or {}),
                 },
             )

@@ -67,6 +67,16 @@ class LLaMAConfig(ModelConfig):
             hidden = self.multiple_of * ((hidden + self.multiple_of - 1) // self.multiple_of)
         return hidden
 
+    @property
+    def max_positions(self) -> int:
+        """The most tokens a sequence may hold.  max_expected_seq_len, except with "ntk" scaling, which stretches
+        the rotation for longer sequences (fms/modules/positions.py:135-168): the reference sets no end to that,
+        here a sequence may grow to rope_scaling["factor"] times max_expected_seq_len (factor 1 if not given)."""
+        scaling = self.rope_scaling or {}
+        if scaling.get("rope_type") == "ntk":
+            return int(self.max_expected_seq_len * float(scaling.get("factor", 1.0)))
+        return self.max_expected_seq_len
+
     def validate(self) -> None:
         problems = []
         if self.nheads <= 0 or self.emb_dim <= 0 or self.nlayers < 0 or self.src_vocab_size <= 0:
@@ -82,13 +92,10 @@ class LLaMAConfig(ModelConfig):
         if self.p_dropout:
             problems.append("p_dropout must be 0: this library only generates")
         kind = (self.rope_scaling or {}).get("rope_type", "regular")
-        if kind == "ntk":
-            # fms/modules/positions.py:135-168, 311-355: the table is chosen by the longest sequence of each call, so
-            # a token's rotation depends on how the tokens were cut into calls and on the rest of the batch
-            problems.append("rope_scaling rope_type 'ntk' is not built: its rotation depends on the length of each "
-                            "call, which a step function over a cache cannot reproduce; use regular or llama3")
-        elif kind not in ("regular", "llama3"):
-            problems.append(f"rope_scaling rope_type {kind!r} is not one of regular, llama3")
+        if kind not in ("regular", "llama3", "ntk"):
+            problems.append(f"rope_scaling rope_type {kind!r} is not one of regular, llama3, ntk")
+        if kind == "ntk" and float((self.rope_scaling or {}).get("factor", 1.0)) < 1.0:
+            problems.append("rope_scaling factor of ntk scaling must be at least 1")
         if problems:
             raise ValueError("invalid LLaMAConfig: " + "; ".join(problems))
 

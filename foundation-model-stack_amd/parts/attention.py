@@ -61,6 +61,10 @@ class MultiHeadAttention(Mixer):
     def state_need(self):
         return None
 
+    @property
+    def graph_safe(self) -> bool:
+        return getattr(self.position_encoder, "graph_safe", True)
+
     def check_step(self, max_position: int) -> None:
         if self.position_encoder is not None:
             self.position_encoder.check_positions(max_position)
@@ -87,7 +91,7 @@ class MultiHeadAttention(Mixer):
         x, row_norm = split_normed(x)
         H, K, D = self.nheads, self.kvheads, self.head_dim
         table = batch.block_tables[cache.group]
-        tables = self.position_encoder.rotary_tables() if self.position_encoder is not None else None
+        tables = self.position_encoder.tables_for_step(batch) if self.position_encoder is not None else None
         cos, sin, rot = tables if tables is not None else (None, None, 0)
         keys, values = (cache.keys, cache.values) if cache.owns else (None, None)
         weight = self.qkv.w["weight"]

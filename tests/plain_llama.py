@@ -82,12 +82,23 @@ def linear(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] =
     return y
 
 
-def rope_frequencies(head_dim: int, theta: float, scaling: Optional[dict] = None) -> torch.Tensor:
-    """fms/modules/positions.py:124-132 (no scaling) and :171-196 (llama3 scaling)."""
-    freqs = 1.0 / (theta ** (torch.arange(0, head_dim, 2)[: head_dim // 2].float() / head_dim))
+def ntk_alpha(length: int, original_length: int) -> int:
+    """fms/modules/positions.py:146-156: ceil(length / original), rounded up to a power of two."""
+    alpha = math.ceil(length / original_length)
+    return int(2 ** math.ceil(math.log(alpha) / math.log(2)))
+
+
+def rope_frequencies(head_dim: int, theta: float, scaling: Optional[dict] = None, length: int = 0, max_len: int = 0) -> torch.Tensor:
+    """fms/modules/positions.py:124-132 (no scaling), :171-196 (llama3 scaling) and :135-168 (ntk scaling: for a
+    call whose longest sequence has `length` tokens, theta times alpha^(D / (D - 2)) with the power of two
+    alpha that stretches the table's `max_len` positions over it; alpha 1 for shorter calls)."""
     scaling = scaling or {}
     kind = scaling.get("rope_type", "regular")
-    if kind == "regular":
+    if kind == "ntk":
+        alpha = ntk_alpha(max(length, 1), max_len)
+        theta = theta * alpha ** (head_dim / (head_dim - 2))
+    freqs = 1.0 / (theta ** (torch.arange(0, head_dim, 2)[: head_dim // 2].float() / head_dim))
+    if kind in ("regular", "ntk"):
         return freqs
     if kind != "llama3":
         raise ValueError(f"plain implementation has no rope_type {kind!r}")
@@ -265,10 +276,11 @@ def forward(
     w = {name: t.float() for name, t in weights.items()}
     tokens = torch.as_tensor(ids, dtype=torch.long)
     positions = torch.arange(len(ids)) + first_position
-    if int(positions[-1]) >= cfg.max_len:
+    stretches = (cfg.rope_scaling or {}).get("rope_type") == "ntk"
+    if int(positions[-1]) >= cfg.max_len and not stretches:
         # tests/modules/test_positions.py:156-168: a position beyond the table raises
         raise IndexError("position beyond max_expected_seq_len")
-    freqs = rope_frequencies(cfg.head_dim, cfg.theta, cfg.rope_scaling)
+    freqs = rope_frequencies(cfg.head_dim, cfg.theta, cfg.rope_scaling, int(positions[-1]) + 1, cfg.max_len)
     x = rs(embedding(w["base_model.embedding.weight"], tokens))
     for i in range(cfg.nlayers):
         p = f"base_model.layers.{i}."

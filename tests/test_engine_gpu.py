@@ -611,6 +611,42 @@ def test_a_type_asked_for_casts_a_checkpoint_stored_in_32_bit(lib, tmp_path):
     check(torch.cat(got), expect(weights16, cfg, ids, "bfloat16"), "bfloat16")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_ntk_scaling(lib, dtype, tmp_path):
+    """fms/modules/positions.py:135-168, 311-355: the rotation's base grows with the longest sequence of a call.  Up
+    to max_expected_seq_len the model is the regular one (tests/modules/test_positions.py:216-241); a longer prompt
+    in one step is rotated with the stretched base throughout, like the reference's call with that prompt; steps
+    run eagerly, because a captured step would keep the table it was captured with."""
+    from fms_amd.engine import Engine
+    from fms_amd.sampling import SamplingParams
+
+    kw = dict(CONFIGS["A"], max_expected_seq_len=64, rope_scaling={"rope_type": "ntk", "factor": 4.0})
+    folder = str(tmp_path / "ntk")
+    lib.write_model_folder(folder, lib.LLaMAConfig(**kw), seed=51, std=0.08, norm_std=0.2)
+    cfg, weights = P.load_model_folder(folder)
+    assert cfg.rope_scaling["rope_type"] == "ntk" and cfg.max_len == 64
+    model = lib.get_model("hf_pretrained", model_path=folder, data_type=dtype)
+    engine = Engine(model, max_tokens=512, max_slots=2)
+    assert not engine.use_graphs and engine.cache.max_seq_len == 256
+    regular = P.PlainConfig(**{**cfg.__dict__, "rope_scaling": {}})
+    short, long_one = tokens_for("A", 64, 52), tokens_for("A", 150, 53)
+    a, b = engine.new_sequence(), engine.new_sequence()
+    got = engine.step([a], [short[:40]], "all")
+    got = torch.cat([got] + [engine.step([a], [[t]], "last") for t in short[40:]])
+    check(got, expect(weights, regular, short, dtype), dtype)  # alpha 1: the regular rotation
+    check(engine.step([b], [long_one], "all"), expect(weights, cfg, long_one, dtype), dtype)  # alpha 4 throughout
+    assert float((P.forward(weights, cfg, long_one) - P.forward(weights, P.PlainConfig(**{**cfg.__dict__, "max_len": 256, "rope_scaling": {}}), long_one)).abs().max()) > 0.05
+    # decoding goes on across the borders where alpha changes (64, 128), eagerly, up to the last position
+    tokens = engine.decode_and_choose([a, b], [1, 2], SamplingParams(do_sample=False))
+    assert len(tokens) == 2 and engine.length(a) == 65
+    engine.end_sequence(a)
+    for _ in range(256 - 151):
+        tokens = engine.decode_and_choose([b], tokens[-1:], SamplingParams(do_sample=False))
+    assert engine.length(b) == 256
+    with pytest.raises(IndexError):
+        engine.step([b], [[1]], "last")
+
+
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_a_meta_checkpoint_runs(lib, folders, name, tmp_path):
     """fms/models/llama.py:618-645: Meta's tensor names (w1 is the gate, w3 the up projection, adjacent rotary

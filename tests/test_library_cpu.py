@@ -282,12 +282,35 @@ def test_the_architecture_tells_a_checkpoints_source():
     assert not hasattr(models, "detect_source")  # the generic loader asks the architecture
 
 
-def test_ntk_scaling_is_refused_with_the_configuration():
-    """fms/modules/positions.py:135-168: the table depends on the length of each call."""
-    with pytest.raises(ValueError, match="ntk"):
-        LLaMAConfig(**TINY, rope_scaling={"rope_type": "ntk"})
-    with pytest.raises(ValueError, match="ntk"):
-        LLaMAConfig.from_hf_dict({**LLaMAConfig(**TINY).to_hf_dict(), "rope_scaling": {"rope_type": "ntk"}})
+def test_ntk_scaling_stretches_the_positions():
+    """fms/modules/positions.py:135-168: alpha is the power of two that covers the call's longest sequence; up to
+    the table's length it is 1.  The configuration lets sequences grow to factor times max_expected_seq_len."""
+    from fms_amd.parts.position import RotaryEncoding, ntk_alpha, rope_frequencies
+
+    for n, want in ((1, 1), (64, 1), (65, 2), (128, 2), (129, 4), (256, 4), (257, 8), (1000, 16)):
+        assert ntk_alpha(n, 64) == want == P.ntk_alpha(n, 64)
+    config = LLaMAConfig(**TINY, rope_scaling={"rope_type": "ntk", "factor": 4.0})
+    assert config.max_positions == 4 * config.max_expected_seq_len
+    assert LLaMAConfig(**TINY, rope_scaling={"rope_type": "ntk"}).max_positions == config.max_expected_seq_len
+    assert LLaMAConfig(**TINY).max_positions == config.max_expected_seq_len
+    back = LLaMAConfig.from_hf_dict(config.to_hf_dict())
+    assert back.rope_scaling == config.rope_scaling and back.max_positions == config.max_positions
+    spec = llama_spec(config)
+    assert spec.max_seq_len == config.max_positions
+    assert spec.positions["rope"].args["max_seq_len"] == config.max_expected_seq_len
+    with pytest.raises(ValueError, match="factor"):
+        LLaMAConfig(**TINY, rope_scaling={"rope_type": "ntk", "factor": 0.5})
+    scaling = {"rope_type": "ntk"}
+    for alpha in (1, 2, 8):
+        torch.testing.assert_close(rope_frequencies(16, 1e4, scaling, alpha), P.rope_frequencies(16, 1e4, scaling, 64 * alpha, 64))
+    torch.testing.assert_close(rope_frequencies(16, 1e4, scaling, 1), rope_frequencies(16, 1e4))
+    rope = RotaryEncoding(16, 1e4, 64, scaling, max_positions=256)
+    assert not rope.graph_safe and RotaryEncoding(16, 1e4, 64, scaling).graph_safe and RotaryEncoding(16, 1e4, 64).graph_safe
+    rope.check_positions(255)
+    with pytest.raises(IndexError):
+        rope.check_positions(256)
+    with pytest.raises(IndexError):
+        RotaryEncoding(16, 1e4, 64, {}, max_positions=256).check_positions(64)  # only ntk stretches
 
 
 def test_schedule_is_data():

@@ -174,6 +174,21 @@ def test_rope_pairings_agree_after_row_permutation():
     torch.testing.assert_close(q_ref.reshape(S, heads, D // 2, 2).transpose(2, 3).reshape(S, heads, D), q_hf)
 
 
+def test_rope_ntk_scaling_reference_vector():
+    """tests/modules/test_positions.py:216-241: up to the table's length ntk scaling changes nothing; for a
+    sequence of twice that length it equals the regular rotation of a base that is 2^(D/(D-2)) times larger."""
+    D, S = 50, 10
+    x = torch.randn(S, 5, D)
+    positions = torch.arange(S)
+    regular = P.rope_rotate(x, positions, P.rope_frequencies(D, 10_000.0))
+    same = P.rope_rotate(x, positions, P.rope_frequencies(D, 10_000.0, {"rope_type": "ntk"}, S, S))
+    torch.testing.assert_close(same, regular)
+    scaled_ratio = 10_000 / 2 ** (D / (D - 2))
+    stretched = P.rope_rotate(x, positions, P.rope_frequencies(D, scaled_ratio, {"rope_type": "ntk"}, S, S // 2))
+    torch.testing.assert_close(stretched, regular)
+    assert [P.ntk_alpha(n, 5) for n in (1, 5, 6, 10, 11, 21)] == [1, 1, 2, 2, 4, 8]
+
+
 def test_rope_llama3_scaling_limits():
     scaling = {
         "rope_type": "llama3",
