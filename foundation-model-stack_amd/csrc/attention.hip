@@ -53,7 +53,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
     const int j = base + threadIdx.x;
     float s = -INFINITY;
     if (j <= pos) {
-      const T* krow = k_cache + (size_t)bt[j / PAGE_TOKENS] * page_elems +
+      const T* krow = k_cache + readable_page(bt[j / PAGE_TOKENS]) * page_elems +
                       ((size_t)kh * PAGE_TOKENS + j % PAGE_TOKENS) * head_dim;
       float dot = 0.f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_f32(krow[d]), dot);
@@ -72,7 +72,7 @@ __global__ void __launch_bounds__(GEN_THREADS)
       const int n = pos - base + 1 < GEN_THREADS ? pos - base + 1 : GEN_THREADS;
       for (int i = 0; i < n; ++i) {
         const int jj = base + i;
-        const T* vrow = v_cache + (size_t)bt[jj / PAGE_TOKENS] * page_elems +
+        const T* vrow = v_cache + readable_page(bt[jj / PAGE_TOKENS]) * page_elems +
                         ((size_t)kh * head_dim + d) * PAGE_TOKENS + jj % PAGE_TOKENS;
         a = fmaf(ps[i], to_f32(*vrow), a);
       }
@@ -255,7 +255,7 @@ __device__ __forceinline__ void attn_wave_pages(WaveState<MAXDT, QT>& st, const 
   if (key_hi < key_lo) return;
   const int page_last = key_hi / PAGE_TOKENS;
   for (int pi = page_first; pi <= page_last; pi += page_step) {
-    const size_t phys = (size_t)bt[pi];
+    const size_t phys = readable_page(bt[pi]);
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
 #pragma unroll
@@ -466,7 +466,7 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
   constexpr int PF = 2;
   bf16x8 kbuf[PF][CH], vbuf[PF][CH];
   auto fetch = [&](int pi, bf16x8 (&kb)[CH], bf16x8 (&vb)[CH]) {
-    const size_t phys = (size_t)bt[pi];
+    const size_t phys = readable_page(bt[pi]);
     const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
     const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
 #pragma unroll
@@ -792,11 +792,11 @@ __device__ __forceinline__ void decode_pages_staged(WaveState<8, 1>& st, const b
   if (first > last) return;
   const size_t head_off = (size_t)kh * PAGE_TOKENS * 128;
   bf16x8 raw[16];
-  size_t phys = (size_t)uniform_load(bt + first);
+  size_t phys = readable_page(uniform_load(bt + first));
   staged_load(raw, k_cache + phys * page_elems + head_off);
   int pi = first;
   for (; pi + stride <= last; pi += stride) {
-    const size_t next = (size_t)uniform_load(bt + pi + stride);
+    const size_t next = readable_page(uniform_load(bt + pi + stride));
     staged_page_step<true>(st, qreg, qpos, qlo, pi * PAGE_TOKENS, raw, v_cache + phys * page_elems + head_off,
                            k_cache + next * page_elems + head_off, buf, scale2);
     phys = next;
@@ -875,7 +875,7 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
                           stage + wave * 8192, scale * LOG2E);
   } else {
     for (int pi = page_lo + wave; pi <= page_hi; pi += n_waves) {
-      const size_t phys = (size_t)uniform_load(bt + pi);
+      const size_t phys = readable_page(uniform_load(bt + pi));
       const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
       const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
       if (MAXDT <= 8) {

@@ -39,6 +39,11 @@ void fmsamd_set_error(const char* fmt, ...);
     }                                                                            \
   } while (0)
 
+// A block-table entry below zero marks a page that is not there: never handed out, or given back by a window.
+// No kernel needs such a page for a key it can see or a token it writes; if the host's bookkeeping is ever
+// wrong, a read goes to page 0 and a write is dropped, instead of leaving the cache's memory.
+__device__ __forceinline__ size_t readable_page(int entry) { return entry < 0 ? 0 : (size_t)entry; }
+
 // --------------------------------------------------------------------------
 // conversions
 // --------------------------------------------------------------------------

@@ -247,7 +247,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
   if (EPI == EPI_ROPE && threadIdx.x < MT * 16) {
     // index data of the rows, fetched while the weights stream
     const int m = threadIdx.x;
-    int pos = 0, seq = -1, page = 0;
+    int pos = 0, seq = -1, page = -1;
     if (m < M) {
       seq = rope.seq_of_token[m];
       pos = rope.positions[m];
@@ -480,7 +480,7 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       }
       if (hh < rope.nheads) {
         out[(size_t)m * ldo + n] = from_f32<OutT>(v);
-      } else if (seq >= 0 && rope.k_cache != nullptr) {
+      } else if (seq >= 0 && rope.k_cache != nullptr && s_page[m] >= 0) {
         const size_t page_elems = (size_t)rope.kvheads * PAGE_TOKENS * D;
         const int in_page = pos % PAGE_TOKENS;
         if (hh < rope.nheads + rope.kvheads) {

@@ -335,10 +335,13 @@ __global__ void __launch_bounds__(256)
     if (hh < rope.nheads) {
       out[(size_t)m * ldo + n] = from_f32<OutT>(v);
     } else if (seq >= 0 && rope.k_cache != nullptr) {
-      const size_t page = (size_t)rope.block_table[(size_t)seq * rope.table_stride + pos / PAGE_TOKENS];
+      const int entry = rope.block_table[(size_t)seq * rope.table_stride + pos / PAGE_TOKENS];
+      const size_t page = readable_page(entry);
       const size_t page_elems = (size_t)rope.kvheads * PAGE_TOKENS * D;
       const int in_page = pos % PAGE_TOKENS;
-      if (hh < rope.nheads + rope.kvheads) {
+      if (entry < 0) {
+        // no page for this token: nothing is written
+      } else if (hh < rope.nheads + rope.kvheads) {
         const int kh = hh - rope.nheads;
         rope.k_cache[page * page_elems + ((size_t)kh * PAGE_TOKENS + in_page) * D + d] = (bf16)v;
       } else {

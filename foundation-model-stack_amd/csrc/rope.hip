@@ -50,7 +50,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const
 
   long page = 0;
   int in_page = pos % PAGE_TOKENS;
-  if (k_cache) page = block_table[(size_t)seq * table_stride + pos / PAGE_TOKENS];
+  if (k_cache) {
+    page = block_table[(size_t)seq * table_stride + pos / PAGE_TOKENS];
+    if (page < 0) k_cache = nullptr, v_cache = nullptr;  // no page for this token: queries only
+  }
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
 
   const int total = (nheads + 2 * kvheads) * half;
