@@ -334,6 +334,39 @@ def sampling_distribution(logits: torch.Tensor, temperature: float, top_k: int) 
     return torch.softmax(scaled, dim=-1)
 
 
+# The seeded draw has no counterpart in the reference (its torch.multinomial takes the global generator,
+# fms/utils/generation.py:326); what follows states this library's definition a second time, on its own: the
+# uniform number of a request's n-th draw is splitmix64 of (request seed + (n + 1) * the golden-ratio constant),
+# its top 24 bits; the request seed is two rounds of the same mixing over (call seed, request index); and the
+# token is the first index at which the cumulative distribution passes the number.
+_M64 = (1 << 64) - 1
+
+
+def _splitmix_finish(z: int) -> int:
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _M64
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _M64
+    return z ^ (z >> 31)
+
+
+def draw_uniform(request_seed: int, n_drawn: int) -> float:
+    return (_splitmix_finish((request_seed + (n_drawn + 1) * 0x9E3779B97F4A7C15) & _M64) >> 40) / float(1 << 24)
+
+
+def seed_of_request(call_seed: int, request_index: int) -> int:
+    return _splitmix_finish((_splitmix_finish(call_seed & _M64) + 0xD1342543DE82EF95 * (request_index + 1)) & _M64) >> 1
+
+
+def inverse_cdf(dist: torch.Tensor, u: float):
+    """(token, distance of u from the nearest edge of the token's interval): the first index whose cumulative
+    probability exceeds u."""
+    cdf = torch.cumsum(dist.double(), 0)
+    tok = int(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True).clamp(max=dist.numel() - 1))
+    while dist[tok] == 0 and tok > 0:  # u at the very end, beyond rounding: the last token with mass
+        tok -= 1
+    lo = float(cdf[tok] - dist[tok].double())
+    return tok, min(u - lo, float(cdf[tok]) - u)
+
+
 def greedy_generate(weights, cfg: PlainConfig, prompt: List[int], n_new: int, stop: Optional[int] = None) -> List[int]:
     """fms/utils/generation.py:287-346 for one row, greedy, recomputing the whole sequence each step."""
     ids = list(prompt)

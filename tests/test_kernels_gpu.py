@@ -486,8 +486,6 @@ def test_argmax(ops):
 
 @pytest.mark.parametrize("vocab,top_k,temperature", [(50, 0, 1.0), (384, 10, 0.8), (5000, 3, 2.0), (128256, 50, 0.7), (300, 1000, 1.0)])
 def test_sampling(ops, vocab, top_k, temperature):
-    from fms_amd.sampling import uniform
-
     torch.manual_seed(10)
     rows = 64
     logits = torch.randn(rows, vocab) * 3
@@ -500,7 +498,7 @@ def test_sampling(ops, vocab, top_k, temperature):
     for r in range(rows):
         p = P.sampling_distribution(logits[r], temperature, top_k).double()
         cdf = torch.cumsum(p, 0)
-        u = uniform(seeds[r], counters[r])
+        u = P.draw_uniform(seeds[r], counters[r])  # the plain implementation's own statement of the generator
         tok = out[r]
         assert p[tok] > 0, "a token outside the kept set was drawn"
         lo = float(cdf[tok] - p[tok])

@@ -289,6 +289,19 @@ def test_bfloat16_roundings_of_the_reference():
     assert torch.equal(P.forward(weights, cfg, ids, storage=torch.float32, rounding="reference"), exact)
 
 
+def test_seeded_draws():
+    """The uniform numbers fill [0, 1) evenly and differ by request and by draw; the inverse CDF picks the token
+    whose interval holds the number."""
+    us = [P.draw_uniform(P.seed_of_request(3, r), n) for r in range(8) for n in range(250)]
+    assert all(0 <= u < 1 for u in us) and len(set(us)) > 1990
+    assert abs(sum(us) / len(us) - 0.5) < 0.03 and abs(sum(u < 0.1 for u in us) / len(us) - 0.1) < 0.03
+    assert P.draw_uniform(5, 9) == P.draw_uniform(5, 9) != P.draw_uniform(5, 10)
+    assert P.seed_of_request(3, 0) != P.seed_of_request(3, 1) != P.seed_of_request(4, 1)
+    dist = torch.tensor([0.0, 0.25, 0.0, 0.5, 0.25, 0.0])
+    assert [P.inverse_cdf(dist, u)[0] for u in (0.0, 0.2, 0.25, 0.7, 0.75, 0.999)] == [1, 1, 3, 3, 4, 4]
+    assert abs(P.inverse_cdf(dist, 0.3)[1] - 0.05) < 1e-9
+
+
 def test_sampling_distribution():
     logits = torch.tensor([1.0, 3.0, 2.0, 3.0, -1.0])
     p = P.sampling_distribution(logits, 0.5, 2)
