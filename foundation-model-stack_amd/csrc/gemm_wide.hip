@@ -1,4 +1,4 @@
-// bfloat16 products y = x W^T for 17 to 64 rows of x, weights [rows, K] with K contiguous.
+// bfloat16 products y = x W^T for 17 to 128 rows of x, weights [rows, K] with K contiguous.
 //
 // With this many rows of x the activations are no longer small beside the weights: a block that owns 16
 // weight rows and all of K (gemm.hip) reads four times as many bytes of x as of W.  Here a block owns 128
@@ -13,6 +13,7 @@
 #define WD_ROWS 128   // weight rows per block
 #define WD_GROUP 128  // k-values per step of the stream
 #define WD_COMPUTE_UNITS 256
+#define WD_MAX_ROWS FMS_SKINNY_MAX_ROWS  // rows of x: eight tiles of 16
 #define WD_DEPTH 4       // steps whose loads are in flight (even)
 #define WD_TILE_LD 132   // floats per row of the block's result tile in LDS: 128 and a shift of the banks
 
@@ -176,21 +177,27 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
         for (int st = 0; st < 4; ++st)
           a[st] = *reinterpret_cast<const bf16x8*>(ws + r * WD_GROUP + (((st * 4 + g) ^ r) & 15) * 8);
-        // all operands of the step first, then the products: a read that waits in front of every product
-        // would pay the LDS latency sixteen times a step
-        bf16x8 b[MT][4];
+        // all operands of four tiles of x first, then their products: a read that waits in front of every
+        // product would pay the LDS latency sixteen times a step
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
+        for (int j0 = 0; j0 < MT; j0 += 4) {
+          constexpr int JT = MT < 4 ? MT : 4;
+          bf16x8 b[JT][4];
 #pragma unroll
-          for (int st = 0; st < 4; ++st) {
-            const int m = j * 16 + r;
-            b[j][st] = *reinterpret_cast<const bf16x8*>(xs + buf * (MT * 16 * WD_GROUP) + m * WD_GROUP +
-                                                        (((st * 4 + g) ^ m) & 15) * 8);
-          }
+          for (int jj = 0; jj < JT; ++jj)
 #pragma unroll
-        for (int j = 0; j < MT; ++j)
+            for (int st = 0; st < 4; ++st) {
+              const int m = (j0 + jj < MT ? j0 + jj : MT - 1) * 16 + r;
+              b[jj][st] = *reinterpret_cast<const bf16x8*>(xs + buf * (MT * 16 * WD_GROUP) + m * WD_GROUP +
+                                                           (((st * 4 + g) ^ m) & 15) * 8);
+            }
 #pragma unroll
-          for (int st = 0; st < 4; ++st) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[st], b[j][st], acc[j], 0, 0, 0);
+          for (int jj = 0; jj < JT; ++jj)
+            if (j0 + jj < MT)
+#pragma unroll
+              for (int st = 0; st < 4; ++st)
+                acc[j0 + jj] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[st], b[jj][st], acc[j0 + jj], 0, 0, 0);
+        }
       }
     }
   }
@@ -432,8 +439,12 @@ static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float
     FMS_WK(2);
   else if (mt == 3)
     FMS_WK(3);
-  else
+  else if (mt == 4)
     FMS_WK(4);
+  else if (mt <= 6)
+    FMS_WK(6);
+  else
+    FMS_WK(8);
 #undef FMS_WK
 }
 
@@ -457,7 +468,7 @@ int wide_product(int epi, const void* x, long ldx, const void* w, const void* bi
                  int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, RowScale scale,
                  RopeEpilogue rope, ResidEpilogue res, void* workspace, long workspace_bytes, hipStream_t stream) {
   const int rows = epi == EPI_GATED ? tile2_offset + N : N;
-  FMS_REQUIRE(M > 16 && M <= 64, "wide product: %d rows (17..64)", M);
+  FMS_REQUIRE(M > 16 && M <= WD_MAX_ROWS, "wide product: %d rows (17..%d)", M, WD_MAX_ROWS);
   const int slices = wide_slices(epi, M, rows, K);
   const int ngroups = ceil_div(K, WD_GROUP);
   const int per_slice = ceil_div(ngroups, slices);

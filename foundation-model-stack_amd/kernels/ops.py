@@ -235,7 +235,7 @@ def qkv_rope_write(
     head_dim: int,
     row_norm: Optional[RowNorm] = None,
 ) -> torch.Tensor:
-    """The fused qkv projection of a decode step (at most 64 rows, bfloat16): x W^T (+ bias), q and k
+    """The fused qkv projection of a decode step (at most 128 rows, bfloat16): x W^T (+ bias), q and k
     rotated, k and v written into their cache pages.  Returns the [M, (H+2K)*D] buffer whose query
     columns hold the rotated queries (its other columns are not written).  Equal to `linear` followed
     by `rope_kv_write`."""
@@ -246,7 +246,7 @@ def qkv_rope_write(
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or tuple(weight.shape) != (N, K) or not weight.is_contiguous():
         raise ValueError(f"qkv_rope_write takes bfloat16 x [M, {K}] and a contiguous bfloat16 weight [{N}, {K}]")
     if M > QKV_ROPE_MAX_ROWS or K % 8 or x.stride(0) % 8 or N % 16:
-        raise ValueError("qkv_rope_write: at most 64 rows, K a multiple of 8, the output row a multiple of 16")
+        raise ValueError(f"qkv_rope_write: at most {QKV_ROPE_MAX_ROWS} rows, K a multiple of 8, the output row a multiple of 16")
     if bias is not None and (bias.shape != (N,) or not bias.is_contiguous()):
         raise ValueError(f"bias must be a contiguous [{N}] tensor")
     _check_batch_index(positions, seq_of_token, block_table, M)
@@ -269,7 +269,7 @@ def qkv_rope_write(
     return out
 
 
-QKV_ROPE_MAX_ROWS = 64
+QKV_ROPE_MAX_ROWS = 128
 
 
 def rope_kv_write(
@@ -417,10 +417,10 @@ def prefill_qblock(nheads: int, kvheads: int, head_dim: int, n_tokens: int) -> i
 # --------------------------------------------------------------------------
 # matrix products
 # --------------------------------------------------------------------------
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 128
 # Up to this many rows the skinny kernel, with the norms, rotation and activation fused into it, beats the
 # vendor library followed by those as kernels of their own.
-SKINNY_FAST_ROWS = 64
+SKINNY_FAST_ROWS = 128
 
 
 def linear(
@@ -434,7 +434,7 @@ def linear(
     """x [M, K] @ weight[N, K]^T (+ bias) -> [M, N].
 
     float32 x float32: the FMA kernel (true 32-bit).  bfloat16 x bfloat16: the weight-streaming
-    skinny kernel up to 64 rows; above that the vendor library (hipBLASLt through torch.matmul,
+    skinny kernels up to 128 rows; above that the vendor library (hipBLASLt through torch.matmul,
     as the reference's nn.Linear does) for bfloat16 output, or this package's MFMA kernels when
     float32 output is wanted or allow_library is False.
     A float32 weight with bfloat16 activations (a tensor the checkpoint keeps in 32-bit) runs the
@@ -453,7 +453,7 @@ def linear(
     out_dtype = out_dtype or x.dtype
     lib = load()
     if row_norm is not None and not (weight.dtype == x.dtype == torch.bfloat16 and M <= SKINNY_FAST_ROWS):
-        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 64 rows")
+        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 128 rows")
     if weight.dtype == torch.float32:
         xf = x if x.dtype == torch.float32 else cast(x.contiguous(), torch.float32)
         bf = bias if bias is None or bias.dtype == torch.float32 else cast(bias, torch.float32)
@@ -505,7 +505,7 @@ def linear_into_stream(
     eps: float,
     row_norm: Optional[RowNorm] = None,
 ):
-    """The last product of a residual branch with what follows it (bfloat16, at most 64 rows):
+    """The last product of a residual branch with what follows it (bfloat16, at most 128 rows):
     resid += x W^T (+ bias) in float32 in place.  Returns (scaled, RowNorm): scaled = resid * norm_weight in
     bfloat16 and the sums of squares of resid's rows by tiles of 16 columns, which a product takes as its
     `row_norm` to read the RMS-normed stream without a norm kernel in between."""
@@ -517,7 +517,7 @@ def linear_into_stream(
     if x.dtype != torch.bfloat16 or weight.dtype != torch.bfloat16 or weight.dim() != 2 or weight.shape[1] != K or not weight.is_contiguous():
         raise ValueError(f"linear_into_stream takes bfloat16 x [M, {K}] and a contiguous bfloat16 weight [N, {K}]")
     if M > SKINNY_FAST_ROWS or K % 8 or x.stride(0) % 8:
-        raise ValueError("linear_into_stream: at most 64 rows, K and the row stride multiples of 8")
+        raise ValueError(f"linear_into_stream: at most {SKINNY_FAST_ROWS} rows, K and the row stride multiples of 8")
     if resid.dtype != torch.float32 or tuple(resid.shape) != (M, N):
         raise ValueError(f"the residual stream is float32 [{M}, {N}]")
     if bias is not None and (bias.shape != (N,) or not bias.is_contiguous()):
@@ -563,7 +563,7 @@ def gated_linear(
                                                    _row_scale(row_norm, M), _ptr(ws), ws_bytes, _stream()))
         return out
     if row_norm is not None:
-        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 64 rows")
+        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 128 rows")
     gu = linear(x, weight, None, allow_library=allow_library)
     return gated_act(gu, bias, activation)
 

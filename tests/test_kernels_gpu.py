@@ -185,7 +185,7 @@ def test_rope_kv_write(ops, dtype, H, K, D, rot):
             assert float(kc[p].abs().sum()) == 0 and float(vc[p].abs().sum()) == 0
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 32, 40, 64])
+@pytest.mark.parametrize("M", [1, 8, 20, 32, 40, 64, 81, 128])
 @pytest.mark.parametrize("H,K,D,rot,E", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 40), (8, 8, 32, 16, 256), (40, 4, 128, 128, 32), (30, 2, 136, 136, 32)])
 def test_qkv_rope_write_equals_the_separate_kernels(ops, M, H, K, D, rot, E):
     """The decode-time fusion (projection + rotation + cache write) against linear followed by rope_kv_write."""
@@ -218,8 +218,12 @@ def test_qkv_rope_write_equals_the_separate_kernels(ops, M, H, K, D, rot, E):
                 ops.rope_kv_write(qkv, *args)
             outs.append(qkv[:, : H * D].cpu().float()[seq >= 0])  # a padding row's queries are never read
             caches.append((kc.cpu().float(), vc.cpu().float()))
-        torch.testing.assert_close(outs[1], outs[0], atol=2e-2, rtol=2e-2)
-        torch.testing.assert_close(caches[1][0], caches[0][0], atol=2e-2, rtol=2e-2)
+        # The separate kernels round the projection to bfloat16 before they rotate it, the fused kernel rotates the
+        # float32 sums: an element that the rotation makes small out of two large ones differs by up to the rounding
+        # of those two, half a bfloat16 step (2^-9 of the largest value) each.
+        step = 2.0 ** -8 * max(float(outs[0].abs().max()), float(caches[0][0].abs().max()))
+        torch.testing.assert_close(outs[1], outs[0], atol=step, rtol=2e-2)
+        torch.testing.assert_close(caches[1][0], caches[0][0], atol=step, rtol=2e-2)
         torch.testing.assert_close(caches[1][1], caches[0][1], atol=2e-2, rtol=2e-2)
         assert float(caches[0][0].abs().sum()) > 0
 
@@ -333,7 +337,7 @@ def test_gemm_f32(ops, M, N, K):
     torch.testing.assert_close(out, (x.double() @ w.double().t() + b.double()).float(), atol=1e-4, rtol=1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 48, 64, 65, 200, 300])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 48, 64, 65, 96, 100, 128, 129, 300])
 @pytest.mark.parametrize("N,K", [(40, 24), (100, 176), (257, 96), (384, 96), (4096 + 16, 512), (20000, 64)])
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(7)
@@ -383,7 +387,7 @@ def test_gemm_bf16_of_widths_that_are_no_multiple_of_8(ops, M, N, K):
         torch.testing.assert_close(out, want, atol=4e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100])
+@pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100, 128, 150])
 @pytest.mark.parametrize("hidden,K", [(44, 24), (77, 40), (176, 64), (1000, 96)])
 def test_gated_linear(ops, M, hidden, K):
     torch.manual_seed(8)
@@ -398,7 +402,7 @@ def test_gated_linear(ops, M, hidden, K):
             torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=4e-2, rtol=2e-2)))
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 64])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 64, 90, 128])
 @pytest.mark.parametrize("N,K,eps", [(48, 24, 1e-5), (96, 176, 1e-6), (4096 + 40, 64, 1e-5), (100, 96, 1e-3), (6144, 32, 1e-5)])
 def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
     """The last product of a branch adds to the float32 stream and leaves the next norm's input; the

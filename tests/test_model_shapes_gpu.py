@@ -2,10 +2,10 @@
 heads) and of the Llama-2-7B shape (as many kv heads as heads), with a vocabulary cut to 4096 so that the plain
 implementation on the CPU stays cheap.  These sizes take other kernels than the tiny configurations do: the
 prefill attention with its head size known at compile time, the decode attention that stages pages in LDS, the
-weight-streaming products with thousands of columns and their variants for 17 to 64 rows, vendor products above
-64 rows.  float32 and bfloat16 against the plain implementation, and bfloat16 against the engine's own float32
-path: whole prompts, the last 32 tokens one by one, ragged batches with reused slots, and decode batches of 5,
-24, 64 and 80 sequences through captured graphs.
+weight-streaming products with thousands of columns and their variants for 17 to 128 rows, vendor products above
+128 rows.  float32 and bfloat16 against the plain implementation, and bfloat16 against the engine's own float32
+path: whole prompts, the last 32 tokens one by one, ragged batches with reused slots, and decode batches of 5
+to 140 sequences through captured graphs.
 
 The cache-consistency check of the reference's benchmark script (scripts/benchmark_inference.py:197-213: a cached
 one-token step against the full recomputation) and its heterogeneous-batch test (tests/utils/test_generate.py:
@@ -128,9 +128,10 @@ def prompt_lengths(n):
     return [(special[i] if i < len(special) else 2 + (53 * i * i + 17 * i) % 250) for i in range(n)]
 
 
-@pytest.mark.parametrize("n_seqs", [5, 24, 64, 80])
+@pytest.mark.parametrize("n_seqs", [5, 24, 64, 80, 128, 140])
 def test_decode_batches_through_graphs(shape, n_seqs):
-    """bfloat16 decode steps of 5, 24, 64 and 80 sequences of unequal lengths, as generation runs them
+    """bfloat16 decode steps of 5 to 140 sequences of unequal lengths (above 128 the products are the vendor's
+    and nothing is fused), as generation runs them
     (decode_and_choose: a captured graph, the token choice inside it), against the engine's float32 path fed
     the same tokens, and both against the plain implementation.  After three steps every third sequence ends."""
     from fms_amd.engine import Engine
