@@ -441,8 +441,12 @@ static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float
     FMS_WK(3);
   else if (mt == 4)
     FMS_WK(4);
-  else if (mt <= 6)
+  else if (mt == 5)
+    FMS_WK(5);
+  else if (mt == 6)
     FMS_WK(6);
+  else if (mt == 7)
+    FMS_WK(7);
   else
     FMS_WK(8);
 #undef FMS_WK
