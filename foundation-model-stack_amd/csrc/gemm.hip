@@ -711,7 +711,7 @@ extern "C" int fmsamd_gemm_skinny_residual_partials(int M, int N, int K) {
   return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
 }
 
-// Bytes of workspace that the products for at most 64 rows need (none up to 16 rows).  rows: all rows of W.
+// Bytes of workspace that the products for at most 128 rows need (none up to 16 rows).  rows: all rows of W.
 extern "C" long fmsamd_gemm_skinny_workspace(int M, int rows, int K) {
   return M > 16 && M <= FMS_SKINNY_MAX_ROWS ? wide_workspace_bytes(M, rows, K) : 0;  // enough for every product of this shape
 }
