@@ -345,10 +345,12 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
         const int limit = GATED && t == 1 ? tile2_offset + n_end : n_end;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          // a row past the block's last is read from the block's first (its sums are never stored), a piece
-          // past K from the row's start (it meets zeros of x)
+          // a row past the block's last is read from the first row of the block's half, which is always there
+          // (the tile's own first row may lie past the end of W when the last block is short; its sums are never
+          // stored), a piece past K from the row's start (it meets zeros of x)
           const int n = nbase + 4 * q + lrow;
-          const size_t at = (size_t)(n < limit ? n : nbase) * K + (kok ? k : 0);
+          const int first = GATED && t == 1 ? tile2_offset + n0 : n0;
+          const size_t at = (size_t)(n < limit ? n : first) * K + (kok ? k : 0);
           wreg[u][t][q] = __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(w + at));
         }
       }
