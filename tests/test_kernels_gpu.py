@@ -488,7 +488,9 @@ def test_argmax(ops):
     assert ops.sample(dev(big), False).cpu().tolist() == big.argmax(-1).tolist()
 
 
-@pytest.mark.parametrize("vocab,top_k,temperature", [(50, 0, 1.0), (384, 10, 0.8), (5000, 3, 2.0), (128256, 50, 0.7), (300, 1000, 1.0)])
+@pytest.mark.parametrize("vocab,top_k,temperature", [(50, 0, 1.0), (384, 10, 0.8), (5000, 3, 2.0), (128256, 50, 0.7), (300, 1000, 1.0),
+                                                     (128256, 0, 0.8), (128256, 10, 1.0), (32000, 256, 1.3), (5000, 300, 1.0),
+                                                     (1031, 1030, 0.9), (64, 5, 1.0), (65, 64, 1.0)])
 def test_sampling(ops, vocab, top_k, temperature):
     torch.manual_seed(10)
     rows = 64
@@ -521,6 +523,38 @@ def test_sampling_ties_at_threshold_survive(ops):
         rng = dev(torch.tensor([[99, c]], dtype=torch.int64))
         seen.add(int(ops.sample(dev(logits), True, 1.0, 2, rng).cpu()[0]))
     assert seen == {3, 50, 77}
+
+
+@pytest.mark.parametrize("vocab", [900, 6000])
+def test_sampling_with_many_equal_values(ops, vocab):
+    """top_k far below the number of equal maxima: every one of them stays, so the draw is uniform over them, in
+    index order.  600 of them fit the kernel's short list of candidates (which it has to put in index order);
+    4000 do not, and the threshold is found over the whole row."""
+    logits = torch.full((1, vocab), 1.5)
+    logits[0, ::3] = -4.0  # a third are low values, the others equal maxima
+    kept = [i for i in range(vocab) if i % 3]
+    for c in range(40):
+        rng = dev(torch.tensor([[5, c]], dtype=torch.int64))
+        tok = int(ops.sample(dev(logits), True, 0.5, 7, rng).cpu()[0])
+        u = P.draw_uniform(5, c)
+        assert tok % 3, "a low value was drawn"
+        assert abs(kept.index(tok) - u * len(kept)) <= 1.5, (c, tok, u)
+
+
+def test_sampling_finds_a_far_value(ops):
+    """One value stands out at each of many places of a large row, the row's ends and the borders of the stretches
+    that the kernel cuts it into among them: with top_k=1 it is drawn whatever the uniform number is."""
+    vocab = 128256
+    places = [0, 1, 63, 64, 8063, 8064, 8065, 16127, 64512, 120959, 120960, 128191, 128192, vocab - 2, vocab - 1]
+    torch.manual_seed(12)
+    logits = torch.randn(len(places), vocab)
+    for r, at in enumerate(places):
+        logits[r, at] = 9.0
+    rng = dev(torch.tensor([[77, r] for r in range(len(places))], dtype=torch.int64))
+    assert ops.sample(dev(logits), True, 0.9, 1, rng).cpu().tolist() == places
+    # and without top_k, at a temperature that leaves the others no mass to speak of
+    rng = dev(torch.tensor([[78, r] for r in range(len(places))], dtype=torch.int64))
+    assert ops.sample(dev(logits * 20), True, 0.05, 0, rng).cpu().tolist() == places
 
 
 def test_kernels_refuse_what_they_cannot_do(ops):
