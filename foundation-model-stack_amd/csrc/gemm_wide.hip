@@ -334,7 +334,7 @@ __global__ void __launch_bounds__(256)
     const int hh = n / D, d = n - hh * D;
     const int pos = rope.positions[m], seq = rope.seq_of_token[m];
     if (hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr && d < rope.rot_dim) {
-      const int tpos = pos < rope.max_pos ? pos : rope.max_pos - 1;  // the host has checked the range
+      const int tpos = pos < 0 ? 0 : (pos < rope.max_pos ? pos : rope.max_pos - 1);  // the host has checked the range
       const float c = rope.cos_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
       const float sn = rope.sin_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
       v = (d & 1) ? sn * partner + c * v : c * v - sn * partner;
@@ -473,9 +473,9 @@ int wide_product(int epi, const void* x, long ldx, const void* w, const void* bi
                  RopeEpilogue rope, ResidEpilogue res, void* workspace, long workspace_bytes, hipStream_t stream) {
   const int rows = epi == EPI_GATED ? tile2_offset + N : N;
   FMS_REQUIRE(M > 16 && M <= WD_MAX_ROWS, "wide product: %d rows (17..%d)", M, WD_MAX_ROWS);
-  const int slices = wide_slices(epi, M, rows, K);
   const int ngroups = ceil_div(K, WD_GROUP);
-  const int per_slice = ceil_div(ngroups, slices);
+  const int per_slice = ceil_div(ngroups, wide_slices(epi, M, rows, K));
+  const int slices = ceil_div(ngroups, per_slice);  // no slice without a step (the kernel divides by its steps)
   const bool itself = slices == 1 && wide_finishes_itself(epi);
   WideOut o{out, ldo, bias, bias != nullptr && bias_dtype == FMS_F32, N, tile2_offset, act, WD_ROWS / 2, 0, scale};
 

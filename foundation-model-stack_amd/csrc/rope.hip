@@ -43,7 +43,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const
   const int seq = seq_of_token[t];
   if (seq < 0) return;  // padding row of a fixed-size batch
   int pos = positions[t];
-  const int tpos = pos < max_pos ? pos : max_pos - 1;  // the host has checked; never read outside the table
+  const int tpos = pos < 0 ? 0 : (pos < max_pos ? pos : max_pos - 1);  // the host has checked; never read outside the table
   const int half = head_dim / 2;
   const int rot_half = rot_dim / 2;
   T* row = qkv + (size_t)t * row_stride;
@@ -140,7 +140,7 @@ __global__ void __launch_bounds__(256)
       T* p = qkv + (size_t)(t0 + tok) * row_stride + (size_t)hh * head_dim + 4 * qd;
       vec4 v = *reinterpret_cast<const vec4*>(p);
       if (cos_t != nullptr) {
-        const int tpos = pos < max_pos ? pos : max_pos - 1;  // the host has checked; never read outside the table
+        const int tpos = pos < 0 ? 0 : (pos < max_pos ? pos : max_pos - 1);  // the host has checked; never read outside the table
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
           const int i = 2 * qd + j;  // the pair (x[2i], x[2i+1])
