@@ -12,7 +12,7 @@
 
 #define SMP_THREADS 1024
 #define SMP_WAVES (SMP_THREADS / WAVE)
-#define SMP_SHORT_K 256       // the largest top_k that is served from a short list of candidates
+#define SMP_SHORT_K 512       // the largest top_k that is served from a short list of candidates
 #define SMP_CANDIDATES 1024   // room in that list: one candidate per thread
 
 __device__ __forceinline__ unsigned int float_key(float x) {
@@ -114,11 +114,11 @@ __device__ __forceinline__ void for_each_value(const float* __restrict__ x, int 
 
 // One block per row.  The row is read in passes whose loads are coalesced.
 //   Always: the largest value.
-//   top_k up to 256: each thread's largest value as well.  At least k values are as large as the k-th largest
+//   top_k up to 512: each thread's largest value as well.  At least k values are as large as the k-th largest
 //   of these 1024, so the k-th largest of the row is no smaller than that bound, and the values at or above
-//   the bound are few (about k) unless many are equal.  A second pass collects them, with their indices, and
-//   the rest happens on that list: the threshold, the order by index, the running sum of the exponentials,
-//   the place where it passes the target.
+//   the bound are few (about k (1 + k / 2048)) unless many are equal.  A second pass collects them, with
+//   their indices, and the rest happens on that list: the threshold, the order by index, the running sum of
+//   the exponentials, the place where it passes the target.
 //   No top_k, a larger one, or a list that overflows: the threshold by a selection over the whole row; then
 //   the sum of the kept exponentials by sixteen stretches of consecutive indices, one per wave; the stretch in
 //   which the running sum passes the target is cut into sixteen again, down to 64 indices, which a wave scans.

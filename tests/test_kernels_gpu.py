@@ -489,7 +489,7 @@ def test_argmax(ops):
 
 
 @pytest.mark.parametrize("vocab,top_k,temperature", [(50, 0, 1.0), (384, 10, 0.8), (5000, 3, 2.0), (128256, 50, 0.7), (300, 1000, 1.0),
-                                                     (128256, 0, 0.8), (128256, 10, 1.0), (32000, 256, 1.3), (5000, 300, 1.0),
+                                                     (128256, 0, 0.8), (128256, 10, 1.0), (32000, 256, 1.3), (5000, 300, 1.0), (128256, 512, 1.0), (49152, 700, 0.9),
                                                      (1031, 1030, 0.9), (64, 5, 1.0), (65, 64, 1.0)])
 def test_sampling(ops, vocab, top_k, temperature):
     torch.manual_seed(10)
