@@ -66,6 +66,7 @@ def generate_requests(
     on_step: Optional[Callable[[int, List[int], List[int]], None]] = None,
     step_times: Optional[List[float]] = None,
     before_step: Optional[Callable[[int, List[int], List[List[int]]], Optional[List[List[int]]]]] = None,
+    after_choice: Optional[Callable] = None,
 ) -> List[List[int]]:
     """New tokens of every request (a stop token is kept, nothing follows it).
 
@@ -73,6 +74,9 @@ def generate_requests(
     cache.max_tokens / cache.max_slots / cache.max_seq_len.  chooser(logits, request_indices,
     counters) -> token ids overrides the built-in sampler (tests use it).  before_step(step, requests, tokens)
     sees the tokens each live request is about to be fed and may return others in their place (as many lists).
+    after_choice(step, requests, logits, tokens) sees the float32 logits [live requests, vocabulary] that the
+    tokens were chosen from and may return other tokens in their place; with it every step is run eagerly, so
+    that its logits are at hand.
     """
     sampling = sampling or SamplingParams(do_sample=False)
     stops: Set[int] = set(int(s) for s in (stop_token_ids or ()))
@@ -89,7 +93,7 @@ def generate_requests(
         seeds = [request_seed(seed, r) for r in request_ids]
         return choose(logits, sampling, seeds, counters).tolist()
 
-    fused = chooser is None and hasattr(engine, "decode_and_choose")
+    fused = chooser is None and after_choice is None and hasattr(engine, "decode_and_choose")
     for batch in plan_batches([len(p) for p in prompts], max_new_tokens, cache.max_tokens, max_batch, cache.max_seq_len):
         slots = {r: engine.new_sequence() for r in batch}
         alive = list(batch)
@@ -113,6 +117,12 @@ def generate_requests(
                 else:
                     logits = engine.step([slots[r] for r in alive], [feed[r] for r in alive], "last")
                     tokens = pick(logits, alive, [len(results[r]) for r in alive])
+                    if after_choice is not None:
+                        given = after_choice(step_no, list(alive), logits, list(tokens))
+                        if given is not None:
+                            if len(given) != len(alive):
+                                raise ValueError("after_choice must return one token per live request")
+                            tokens = [int(t) for t in given]
                 if step_times is not None:
                     step_times.append(time.time() - t0)
                 if on_step is not None:
@@ -186,6 +196,11 @@ def generate(
     reference (fms/utils/generation.py:295-296), with the tokens about to be fed as a tensor [rows alive, n]
     (left-padded with pad_token_id or 0 where the rows differ in length) and the extra_kwargs; the tokens it
     returns are fed instead (the same shape; padding places are ignored).
+    post_iteration_hook(token_position, logits, next_val, kwargs) -> (next_val, kwargs) is called after every choice,
+    as in the reference (fms/utils/generation.py:328-331): token_position counts from the padded prompt's width,
+    logits [B, V] are what the choice was made from (divided by the temperature and cut to top_k when sampling),
+    next_val [B, 1] the chosen tokens; the tokens it returns go on.  Rows that have ended show -inf logits and the
+    fill token.  With this hook every step runs eagerly (its logits have to be at hand).
     """
     from ..engine import Engine  # late import: engine imports the kernels
 
@@ -201,10 +216,10 @@ def generate(
     engine = model if isinstance(model, Engine) else default_engine(model, prompts, max_new_tokens)
     times: List[float] = []
     start = time.time()
+    state = {"kwargs": dict(extra_kwargs or {})}  # the kwargs that the reference threads through both hooks
+    pad = pad_token_id if pad_token_id is not None else 0
     before = None
     if prepare_model_inputs_hook is not None:
-        pad = pad_token_id if pad_token_id is not None else 0
-        state = {"kwargs": dict(extra_kwargs or {})}
 
         def before(step, alive, tokens):
             width = max(len(t) for t in tokens)
@@ -212,9 +227,30 @@ def generate(
             ids, state["kwargs"] = prepare_model_inputs_hook(step, ids, state["kwargs"])
             return [row[width - len(t):] for row, t in zip(ids.tolist(), tokens)]
 
-    hook = None
+    after = None
     if post_iteration_hook is not None:
-        hook = lambda step, alive, tokens: post_iteration_hook(step, alive, tokens)  # noqa: E731
+        fill_token = eos_token_id if eos_token_id is not None else pad
+        n_rows, prompt_length = ids2d.shape
+
+        def after(step, alive, logits, tokens):
+            # fms/utils/generation.py:328-331: (token position, the logits the choice was made from, next_val
+            # [B, 1], kwargs) -> (next_val, kwargs).  With sampling the reference's logits are divided by the
+            # temperature and, with top_k, set to -inf below the k-th largest (:317-323).  Rows that have ended
+            # (the reference keeps feeding them) show -inf everywhere and the fill token.
+            shown = logits.float()
+            if do_sample:
+                shown = shown / temperature
+                if top_k:
+                    kth = torch.topk(shown, min(int(top_k), shown.shape[-1])).values[:, [-1]]
+                    shown = shown.masked_fill(shown < kth, float("-inf"))
+            full = torch.full((n_rows, shown.shape[-1]), float("-inf"), dtype=shown.dtype, device=shown.device)
+            rows = torch.tensor(alive, dtype=torch.long, device=shown.device)
+            full[rows] = shown
+            next_val = torch.full((n_rows, 1), fill_token, dtype=ids2d.dtype, device=shown.device)
+            next_val[rows, 0] = torch.tensor(tokens, dtype=ids2d.dtype, device=shown.device)
+            next_val, state["kwargs"] = post_iteration_hook(step + prompt_length, full, next_val, state["kwargs"])
+            return [int(t) for t in next_val.reshape(n_rows, -1)[rows, 0].tolist()]
+
     new = generate_requests(
         engine,
         prompts,
@@ -222,9 +258,9 @@ def generate(
         sampling=SamplingParams(do_sample=do_sample, temperature=temperature, top_k=top_k or 0),
         stop_token_ids=None if eos_token_id is None else [eos_token_id],
         seed=seed,
-        on_step=hook,
         step_times=times if timing == "per-token" else None,
         before_step=before,
+        after_choice=after,
     )
     if timing == "e2e":
         if engine.device.type == "cuda":

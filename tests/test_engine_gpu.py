@@ -290,6 +290,30 @@ def test_greedy_generation_through_the_entry_point(lib, folders, name):
                    extra_kwargs={"note": "kept"})
     assert out.tolist()[len(prompts[0]) :] == P.greedy_generate(weights, cfg, prompts[1][-len(prompts[0]) :], 4)
     assert calls[0] == (0, (1, len(prompts[0])), "kept") and calls[1] == (1, (1, 1), "kept") and len(calls) == 4
+    # the reference's hook after every choice (fms/utils/generation.py:328-331): token position, the logits the
+    # choice was made from [B, V], next_val [B, 1] and the kwargs; what it returns is what goes on.  Here it
+    # checks what it is shown and forces the second request's third token.
+    shown = []
+
+    def force(position, logits, next_val, kwargs):
+        shown.append((position, tuple(logits.shape), tuple(next_val.shape), next_val[:, 0].tolist(), kwargs.get("note")))
+        assert logits.argmax(-1).tolist() == next_val[:, 0].tolist()
+        if position == 20 + 2:
+            next_val = next_val.clone()
+            next_val[1, 0] = prompts[1][0]
+        return next_val, kwargs
+
+    hooked = generate(model, ids, max_new_tokens=5, do_sample=False, extra_kwargs=dict(extra, note="kept"), post_iteration_hook=force)
+    assert [s[0] for s in shown] == [20, 21, 22, 23, 24]
+    assert all(s[1] == (3, cfg.vocab) and s[2] == (3, 1) and s[4] == "kept" for s in shown)
+    for b, (p, w) in enumerate(zip(prompts, want)):
+        row = hooked[b].tolist()[20:]
+        if b != 1:
+            assert row == w[:5]
+        else:
+            forced = p + w[:2] + [p[0]]
+            assert row[:2] == w[:2] and row[2] == p[0]
+            assert row[3:] == P.greedy_generate(weights, cfg, forced, 2)
     # a stop token ends its own request only
     stop = want[1][3]
     out = generate(model, ids, max_new_tokens=16, do_sample=False, extra_kwargs=extra, eos_token_id=stop)

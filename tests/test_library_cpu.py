@@ -550,6 +550,27 @@ def test_loop_lets_a_hook_change_what_is_fed():
         generate_requests(FakeEngine(), [[1]], max_new_tokens=2, chooser=argmax_chooser, before_step=lambda s, r, t: [])
 
 
+def test_loop_lets_a_hook_see_the_logits_and_change_the_choice():
+    """after_choice sees the logits of the live requests and the tokens chosen from them, and may put others in
+    their place (the reference's post_iteration_hook, fms/utils/generation.py:328-331, reaches the loop through it)."""
+    engine = FakeEngine()
+    seen = []
+
+    def hook(step, requests, logits, tokens):
+        seen.append((step, list(requests), tuple(logits.shape), list(tokens)))
+        assert logits.argmax(-1).tolist() == tokens
+        if step == 1:
+            return [70 for _ in tokens]  # the mock counts on from 70
+        return None
+
+    out = generate_requests(engine, [[10, 11], [20], [30]], max_new_tokens=3, chooser=argmax_chooser, stop_token_ids=[31],
+                            after_choice=hook)
+    assert out == [[12, 70, 71], [21, 70, 71], [31]]
+    assert seen == [(0, [0, 1, 2], (3, 256), [12, 21, 31]), (1, [0, 1], (2, 256), [13, 22]), (2, [0, 1], (2, 256), [71, 71])]
+    with pytest.raises(ValueError):
+        generate_requests(FakeEngine(), [[1]], max_new_tokens=2, chooser=argmax_chooser, after_choice=lambda s, r, l, t: [])
+
+
 def test_loop_runs_as_many_batches_as_the_requests_need():
     engine = FakeEngine(max_tokens=64 * 2, max_slots=2)
     prompts = [[i] for i in range(7)]
