@@ -64,9 +64,19 @@ def get_model(
     source: Optional[str] = None,
     device_type: str = "cuda",
     data_type: Union[None, str, torch.dtype] = None,
+    distributed_strategy: Optional[str] = None,
+    checkpoint_sharding: Optional[str] = None,
+    group=None,
     random_seed: int = 0,
     **kwargs,
 ) -> DecoderModel:
+    """The reference's get_model (fms/models/__init__.py:298-309) on this library: architecture and variant from
+    the registry (or "hf_pretrained"/"hf_configured" and a model folder), weights from `model_path` named as
+    `source` says, on the GPU, in `data_type` (the checkpoint's type if none is given); further keyword arguments
+    override fields of the configuration.  distributed_strategy, checkpoint_sharding and group are the reference's
+    parameters for several GPUs: this library runs on one, so anything but None is refused."""
+    if distributed_strategy is not None or checkpoint_sharding is not None or group is not None:
+        raise NotImplementedError("fms_amd runs a model on one GPU: distributed_strategy, checkpoint_sharding and group must be None")
     dtype = resolve_dtype(data_type)
     if architecture in ("hf_pretrained", "hf_configured"):
         # fms/models/__init__.py:88-98: the folder may come as `variant` or as `model_path`, not both

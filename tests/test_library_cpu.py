@@ -98,6 +98,9 @@ def test_registry():
         fms_amd.get_model("no_such_architecture", "x")
     with pytest.raises(ValueError):
         fms_amd.get_model("llama", "micro", data_type="int7")
+    # the reference's parameters for several GPUs are known by name and refused, not taken for configuration fields
+    with pytest.raises(NotImplementedError):
+        fms_amd.get_model("llama", "micro", distributed_strategy="tp")
     assert variant_config("llama", "micro", nlayers=2).nlayers == 2
     # a model folder's architecture comes from its config.json
     from fms_amd.architectures import architecture_for_hf
@@ -662,6 +665,55 @@ def test_char_tokenizer():
         tok.convert_tokens_to_ids("AB")
     with pytest.raises(RuntimeError):
         get_tokenizer("/no/such/tokenizer")
+    # the Hugging Face arguments of the reference's interface (fms/utils/tokenizers.py:37-64)
+    assert tok.encode("AB", add_special_tokens=True) == [2, 65, 66]
+    assert tok.decode([2, 65, 66, 3]) == "AB" and tok.decode([2, 65, 3], skip_special_tokens=False) == "\x02A\x03"
+    assert isinstance(get_tokenizer("char_tokenizer", style="fms"), CharTokenizer)
+    with pytest.raises(RuntimeError):
+        get_tokenizer("char_tokenizer", style="sentencepiece")  # no such file
+    with pytest.raises(RuntimeError):
+        get_tokenizer("char_tokenizer", style="no_such_style")
+
+
+def test_file_tokenizers_have_the_reference_interface(tmp_path):
+    """A sentencepiece model and a tokenizer.json, both made here from a few words: encode/decode with the
+    reference's arguments and the four calls its script makes (scripts/inference.py:179-181, 232-234)."""
+    from fms_amd.tokenizers import get_tokenizer
+
+    text = "the cat sat on the mat and the dog sat on the log"
+    spm = pytest.importorskip("sentencepiece")
+    corpus = tmp_path / "corpus.txt"
+    corpus.write_text("\n".join([text, "a cat and a dog", "the log and the mat"] * 20))
+    spm.SentencePieceTrainer.train(input=str(corpus), model_prefix=str(tmp_path / "tiny"), vocab_size=40, model_type="bpe",
+                                   bos_id=1, eos_id=2, unk_id=0, minloglevel=2)
+    for style in (None, "sentencepiece"):
+        tok = get_tokenizer(str(tmp_path / "tiny.model"), style=style)
+        assert (tok.bos_token_id, tok.eos_token_id) == (1, 2) and tok.vocab_size() == 40
+        pieces = tok.tokenize("the cat sat")
+        ids = tok.convert_tokens_to_ids(pieces)
+        assert ids == tok.encode("the cat sat") and tok.encode("the cat sat", add_special_tokens=True) == [1] + ids
+        assert tok.convert_ids_to_tokens(torch.tensor(ids)) == pieces and isinstance(tok.convert_tokens_to_ids(pieces[0]), int)
+        assert tok.convert_tokens_to_string(pieces) == "the cat sat" == tok.decode([1] + ids + [2])
+
+    tokenizers = pytest.importorskip("tokenizers")
+    words = sorted(set(text.split()))
+    vocab = {"<s>": 0, "</s>": 1, "<unk>": 2, **{w: i + 3 for i, w in enumerate(words)}}
+    tk = tokenizers.Tokenizer(tokenizers.models.WordLevel(vocab, unk_token="<unk>"))
+    tk.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    tk.add_special_tokens(["<s>", "</s>"])
+    folder = tmp_path / "hf"
+    folder.mkdir()
+    tk.save(str(folder / "tokenizer.json"))
+    for name, style in ((str(folder), None), (str(folder), "hf"), (str(folder / "tokenizer.json"), None)):
+        tok = get_tokenizer(name, style=style)
+        assert (tok.bos_token_id, tok.eos_token_id) == (0, 1) and tok.vocab_size() == len(vocab)
+        pieces = tok.tokenize("the dog sat")
+        assert pieces == ["the", "dog", "sat"]
+        ids = tok.convert_tokens_to_ids(pieces)
+        assert ids == [vocab[w] for w in pieces] == tok.encode("the dog sat") and tok.convert_tokens_to_ids("dog") == vocab["dog"]
+        assert tok.encode("the dog sat", add_special_tokens=True) == [0] + ids
+        assert tok.convert_ids_to_tokens(ids) == pieces and tok.convert_tokens_to_string(pieces) == "the dog sat"
+        assert tok.decode([0] + ids + [1]) == "the dog sat"
 
 
 def test_command_line_refusals(capsys):
