@@ -67,6 +67,17 @@ class DecoderModel(Part):
         for part in self.positions.values():
             part.finalize(self.device, self.dtype)
 
+    def get_config(self):
+        """The configuration the model was built from (the reference's LLaMA.get_config, fms/models/llama.py:380-381)."""
+        return self.config
+
+    def __call__(self, input_ids: torch.Tensor, last_n_tokens: int = 0, **kwargs) -> torch.Tensor:
+        """Called on token ids as the reference's model is: float32 logits [B, S, V] without a cache kept
+        (generation.logits has the details).  Generation does not come through here: it steps an Engine."""
+        from ..generation import logits
+
+        return logits(self, input_ids, last_n_tokens=last_n_tokens, **kwargs)
+
     # ---- one pass over the tokens of a step --------------------------------
     def forward(self, batch, cache: SequenceCache) -> torch.Tensor:
         """float32 logits [n wanted rows, vocab] of the tokens in `batch`; the cache is extended in place."""

@@ -280,6 +280,51 @@ def generate(
     return result
 
 
+def logits(model, input_ids: torch.Tensor, last_n_tokens: int = 0, extra_kwargs: Optional[dict] = None, **kwargs) -> torch.Tensor:
+    """What the reference's model returns when it is called on token ids without a cache
+    (fms/models/llama.py:425-450): float32 logits [B, S, V] of a rectangular batch ([S, V] for a 1-D input), or of
+    the last `last_n_tokens` places only.  Rows padded by pad_input_ids come with its kwargs (as extra_kwargs or as
+    keyword arguments, the way the reference's model takes `mask` and `position_ids`); a padding place holds zeros.
+    """
+    from ..engine import Engine  # late import: engine imports the kernels
+
+    if not isinstance(input_ids, torch.Tensor) or input_ids.dim() not in (1, 2):
+        raise TypeError("input_ids must be a Tensor [S] or [B, S]")
+    if last_n_tokens < 0:
+        raise ValueError("last_n_tokens counts places from the end: 0 (all) or more")
+    extra = dict(extra_kwargs or {})
+    extra.update(kwargs)
+    if extra.get("use_cache") or extra.get("past_key_value_states") is not None:
+        raise NotImplementedError("a call on token ids keeps no cache: sequences that go on are stepped through an Engine")
+    is_batch = input_ids.dim() > 1
+    ids2d = input_ids if is_batch else input_ids.unsqueeze(0)
+    rows = _real_tokens(ids2d.cpu(), extra)
+    side = extra.get("padding_side", "left")
+    width = ids2d.shape[1]
+    keep = width if last_n_tokens == 0 else min(last_n_tokens, width)
+    # the wanted places of a row, as places among its real tokens (a place that is padding has no logits)
+    wanted = []
+    for tokens in rows:
+        offset = width - len(tokens) if side == "left" else 0  # where the row's first real token sits
+        wanted.append([p - offset for p in range(width - keep, width) if 0 <= p - offset < len(tokens)])
+    engine = model if isinstance(model, Engine) else default_engine(model, rows, 0)
+    slots = [engine.new_sequence() for _ in rows]
+    try:
+        flat = engine.step(slots, rows, wanted)
+    finally:
+        for slot in slots:
+            engine.end_sequence(slot)
+    out = torch.zeros(len(rows), keep, flat.shape[-1], dtype=flat.dtype, device=flat.device)
+    at = 0
+    for b, (tokens, places) in enumerate(zip(rows, wanted)):
+        if places:
+            offset = width - len(tokens) if side == "left" else 0
+            first = places[0] + offset - (width - keep)
+            out[b, first : first + len(places)] = flat[at : at + len(places)]
+            at += len(places)
+    return out if is_batch else out[0]
+
+
 def default_engine(model, prompts, max_new_tokens):
     """An engine for `model` with room for these requests, kept on the model and reused while it is large enough."""
     from ..engine import Engine

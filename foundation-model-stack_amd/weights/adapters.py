@@ -36,6 +36,17 @@ def register_adapter(architecture: str, source: str, step_names: List[str]) -> N
     sources[source] = list(step_names)
 
 
+def extend_adapter(architecture: str, source: str, step_names: List[str]) -> None:
+    """Further steps behind those a source already has (fms/utils/serialization.py:104-148): the source must be
+    registered, and so must the steps."""
+    if source not in _adapters.get(architecture, {}):
+        raise KeyError(f"adapter {source!r} of {architecture!r} must be registered before it is extended")
+    missing = [s for s in step_names if s not in _steps.get(architecture, {})]
+    if missing:
+        raise KeyError(f"adapter {source!r} of {architecture!r} is extended by unknown steps {missing}")
+    _adapters[architecture][source] = _adapters[architecture][source] + list(step_names)
+
+
 def list_sources(architecture: str) -> List[str]:
     return sorted(_adapters.get(architecture, {}))
 
@@ -56,6 +67,15 @@ def get_adapter(architecture: str, source: Optional[str]) -> Step:
         return sd
 
     return run
+
+
+def get_adapted(architecture: str, source: Optional[str], state_dict: Mapping[str, torch.Tensor],
+                adapter_kwargs: Optional[Mapping] = None) -> Mapping[str, torch.Tensor]:
+    """A state dict in the model's own names and layouts (fms/utils/serialization.py:292-317); an empty one is
+    handed back as it is.  Steps that need the model's sizes read them from adapter_kwargs["model_config"]."""
+    if not len(state_dict):
+        return state_dict
+    return get_adapter(architecture, source)(state_dict, **dict(adapter_kwargs or {}))
 
 
 # ---- steps shared by decoder architectures -----------------------------------

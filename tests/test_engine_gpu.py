@@ -324,6 +324,45 @@ def test_greedy_generation_through_the_entry_point(lib, folders, name):
         assert all(t == stop for t in row[cut:])
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_a_call_on_token_ids_gives_the_logits_of_whole_sequences(lib, folders, name):
+    """The model called the way the reference's is (fms/models/llama.py:425-450, no cache): one sequence, a padded
+    batch with the kwargs of pad_input_ids, and the last n places only (headless.py:24-27)."""
+    from fms_amd.generation import pad_input_ids
+
+    cfg, weights = plain(folders, name)
+    model = get(lib, folders, name, "float32")
+    assert model.get_config() is model.config
+    prompts = [tokens_for(name, n, 60 + n) for n in (9, 4, 13)]
+    want = [P.forward(weights, cfg, p) for p in prompts]
+    one = model(torch.tensor(prompts[0]))
+    assert tuple(one.shape) == (9, cfg.vocab)
+    torch.testing.assert_close(one.cpu(), want[0], atol=2e-4, rtol=1e-3)
+    torch.testing.assert_close(model(torch.tensor(prompts[0]), last_n_tokens=2).cpu(), want[0][-2:], atol=2e-4, rtol=1e-3)
+    for side in ("left", "right"):
+        ids, extra = pad_input_ids([torch.tensor(p) for p in prompts], min_pad_length=15, padding_side=side)
+        out = model(ids, **extra).cpu()
+        assert tuple(out.shape) == (3, 15, cfg.vocab)
+        for b, (p, w) in enumerate(zip(prompts, want)):
+            first = 15 - len(p) if side == "left" else 0
+            torch.testing.assert_close(out[b, first : first + len(p)], w, atol=2e-4, rtol=1e-3)
+            rest = torch.cat((out[b, :first], out[b, first + len(p) :]))
+            assert float(rest.abs().max()) == 0.0 if rest.numel() else True
+        last = model(ids, last_n_tokens=3, **extra).cpu()
+        assert tuple(last.shape) == (3, 3, cfg.vocab)
+        for b, (p, w) in enumerate(zip(prompts, want)):
+            if side == "left":
+                torch.testing.assert_close(last[b], w[-3:], atol=2e-4, rtol=1e-3)
+            else:  # the last three places of the padded row: real only where the row is long enough
+                real = max(0, len(p) - 12)
+                if real:
+                    torch.testing.assert_close(last[b, :real], w[len(p) - real :], atol=2e-4, rtol=1e-3)
+                assert float(last[b, real:].abs().max()) == 0.0 if real < 3 else True
+    with pytest.raises(NotImplementedError):
+        model(torch.tensor(prompts[0]), use_cache=True)
+    assert getattr(model, "_default_engine").cache.live_slots() == []
+
+
 def test_bfloat16_generation_follows_the_plain_one(lib, folders):
     from fms_amd.generation import generate_requests
     from fms_amd.engine import Engine

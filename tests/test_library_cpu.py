@@ -200,6 +200,36 @@ def test_meta_adapter_names_and_fusion():
         get_adapter("llama", "no_such_source")
 
 
+def test_adapters_are_registered_extended_and_applied_by_name():
+    """fms/utils/serialization.py:27-148, 292-317: steps and sources are registered once; an existing source can be
+    given further steps; get_adapted applies a source's steps to a state dict and hands an empty one back."""
+    from fms_amd.weights import extend_adapter, get_adapted, list_sources, register_adapter, register_adapter_step
+
+    arch = "toy_adapters"
+    register_adapter_step(arch, "prefix", lambda sd, **kw: {"m." + k: v for k, v in sd.items()})
+    register_adapter_step(arch, "double", lambda sd, factor=2, **kw: {k: v * factor for k, v in sd.items()})
+    with pytest.raises(KeyError):
+        register_adapter_step(arch, "prefix", lambda sd, **kw: sd)
+    register_adapter(arch, "theirs", ["prefix"])
+    with pytest.raises(KeyError):
+        register_adapter(arch, "theirs", ["prefix"])
+    with pytest.raises(KeyError):
+        register_adapter(arch, "other", ["no_such_step"])
+    assert list_sources(arch) == ["theirs"] and list_sources("no_such_architecture") == []
+    sd = {"w": torch.ones(2)}
+    assert list(get_adapted(arch, "theirs", sd, {})) == ["m.w"]
+    extend_adapter(arch, "theirs", ["double"])
+    out = get_adapted(arch, "theirs", sd, {"factor": 3})
+    assert list(out) == ["m.w"] and out["m.w"].tolist() == [3.0, 3.0]
+    with pytest.raises(KeyError):
+        extend_adapter(arch, "no_such_source", ["double"])
+    with pytest.raises(KeyError):
+        extend_adapter(arch, "theirs", ["no_such_step"])
+    empty = {}
+    assert get_adapted(arch, "theirs", empty, {}) is empty
+    assert get_adapted(arch, None, sd, {}) is sd and get_adapted(arch, "fms", sd, None) is sd
+
+
 def test_kept_dtypes():
     assert kept_dtype(torch.bfloat16, "float", torch.bfloat16) == torch.bfloat16
     assert kept_dtype(torch.float16, "float", torch.bfloat16) == torch.bfloat16
