@@ -57,6 +57,16 @@ def read_model_folder_config(model_path: str):
     raise ValueError(f"{cfg_file} names no architecture (neither 'architectures' nor 'architecture')")
 
 
+def _gpu_device(device_type) -> torch.device:
+    device = torch.device(device_type if ":" in str(device_type) or device_type != "cuda" else "cuda:0")
+    if device.type != "cuda":
+        raise RuntimeError("fms_amd models run on the GPU only (device_type='cuda'); there is no CPU path")
+    if not torch.cuda.is_available():  # before anything is allocated: the message is this library's, not the runtime's
+        raise RuntimeError("fms_amd models run on an AMD GPU, and this machine shows none to PyTorch "
+                           "(torch.cuda.is_available() is False); there is no CPU path")
+    return device
+
+
 def get_model(
     architecture: str,
     variant: Optional[str] = None,
@@ -97,12 +107,7 @@ def get_model(
             raise KeyError(f"a variant of {architecture} is needed")
         config = variant_config(architecture, variant, **kwargs)
 
-    device = torch.device(device_type if ":" in str(device_type) or device_type != "cuda" else "cuda:0")
-    if device.type != "cuda":
-        raise RuntimeError("fms_amd models run on the GPU only (device_type='cuda'); there is no CPU path")
-    if not torch.cuda.is_available():  # before anything is allocated: the message is this library's, not the runtime's
-        raise RuntimeError("fms_amd models run on an AMD GPU, and this machine shows none to PyTorch "
-                           "(torch.cuda.is_available() is False); there is no CPU path")
+    device = _gpu_device(device_type)
 
     ckpt_dtype = None
     if model_path is not None:
@@ -130,6 +135,32 @@ def get_model(
         init_random(model, random_seed, device)
     model.finalize_all(device)
     return model
+
+
+def from_config(config: ModelConfig, architecture: str = "llama", data_type: Union[None, str, torch.dtype] = "bfloat16",
+                device_type: str = "cuda", random_seed: int = 0, **kwargs) -> DecoderModel:
+    """A model of `config` with random weights (keyword arguments replace fields of the configuration): what the
+    reference's `LLaMA(config, **kwargs)` followed by `reset_parameters()` gives (fms/models/llama.py:362-394),
+    with this library's random-weights rule (every tensor a function of the seed and its name)."""
+    arch = get_architecture(architecture)
+    if not isinstance(config, arch.config_class):
+        raise TypeError(f"architecture {architecture} is configured by {arch.config_class.__name__}, not {type(config).__name__}")
+    config = config.updated(**kwargs) if kwargs else config
+    dtype = resolve_dtype(data_type) or torch.float32
+    device = _gpu_device(device_type)
+    model = DecoderModel(arch.build_spec(config), dtype, config=config)
+    model.architecture = arch.name
+    init_random(model, random_seed, device)
+    model.finalize_all(device)
+    return model
+
+
+def LLaMA(config=None, **kwargs) -> DecoderModel:
+    """The reference's constructor by its name: `LLaMA(config)` or `LLaMA(emb_dim=..., nlayers=...)`, random weights;
+    `data_type`, `device_type` and `random_seed` as in from_config."""
+    from .config import LLaMAConfig
+
+    return from_config(config if config is not None else LLaMAConfig(), "llama", **kwargs)
 
 
 def write_model_folder(

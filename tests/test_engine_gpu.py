@@ -363,6 +363,22 @@ def test_a_call_on_token_ids_gives_the_logits_of_whole_sequences(lib, folders, n
     assert getattr(model, "_default_engine").cache.live_slots() == []
 
 
+def test_a_model_from_a_configuration_alone(lib):
+    """The reference's `LLaMA(config, **kwargs)` (fms/models/llama.py:362-378): a model with random weights from a
+    configuration; the same seed gives the weights that get_model gives the same variant."""
+    from fms_amd.architectures import variant_config
+
+    cfg = variant_config("llama", "micro", nlayers=2)
+    ids = torch.tensor([5, 17, 3, 200, 9])
+    a = lib.LLaMA(cfg, data_type="float32", random_seed=3)(ids)
+    b = lib.get_model("llama", "micro", data_type="float32", random_seed=3, nlayers=2)(ids)
+    c = lib.LLaMA(variant_config("llama", "micro"), nlayers=2, data_type="float32", random_seed=4)(ids)
+    assert tuple(a.shape) == (5, 256) and torch.equal(a, b) and not torch.equal(a, c)
+    assert lib.LLaMA(nlayers=1, emb_dim=64, nheads=2, src_vocab_size=50).get_config().nlayers == 1
+    with pytest.raises(TypeError):
+        lib.from_config(lib.ModelConfig())
+
+
 def test_bfloat16_generation_follows_the_plain_one(lib, folders):
     from fms_amd.generation import generate_requests
     from fms_amd.engine import Engine
