@@ -175,7 +175,7 @@ def generate(
     top_k: int = 10,
     do_sample: bool = True,
     num_beams: int = 1,
-    use_cache: bool = True,
+    use_cache: bool = False,
     contiguous_cache: bool = False,
     eos_token_id: Optional[int] = None,
     pad_token_id: Optional[int] = None,
