@@ -39,7 +39,17 @@ def main() -> int:
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="run one phase only (for profiling); the record then lacks the other")
+    # the workload options of the reference's scripts/benchmark_inference.py:70-87, by their names
+    ap.add_argument("--seq_len", type=int, default=None, help="every prompt of the decode batches has this many tokens")
+    ap.add_argument("--batch_size", type=int, default=None, help="the same as --batch")
+    ap.add_argument("--max_new_tokens", type=int, default=None, help="the same as --steps: decode steps that are timed")
     args = ap.parse_args()
+    if args.seq_len is not None:
+        args.prompt_min = args.prompt_max = args.seq_len
+    if args.batch_size is not None:
+        args.batch = args.batch_size
+    if args.max_new_tokens is not None:
+        args.steps = args.max_new_tokens
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print(f"bench.py measures one GPU: this library runs on a single MI355X, --gpus {args.gpus} is not supported")
         return 2
