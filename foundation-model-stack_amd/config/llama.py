@@ -5,7 +5,8 @@ Fields and defaults are those of ``LLaMAConfig`` (fms/models/llama.py:42-62).
 reference's parameter builder does (fms/models/hf/config_utils/param_builders.py:18-58,
 512-546), except that the feed-forward width is carried as the integer that
 config.json gives instead of being rebuilt from a float ratio, and that keys
-the reference silently ignores (``head_dim``, ``hidden_act``) are checked.
+the reference silently ignores are not: ``head_dim`` is checked and ``hidden_act``
+becomes ``activation_fn``.
 """
 
 from __future__ import annotations
@@ -16,6 +17,8 @@ from typing import Optional
 from .base import ModelConfig
 
 HF_ARCHITECTURES = ("LlamaForCausalLM",)
+# the activation functions the reference knows by name (fms/utils/activation.py:14-24)
+ACTIVATION_NAMES = ("swish", "silu", "gelu", "gelu-tanh", "gelu_pytorch_tanh", "mish", "relu", "sigmoid", "tanh")
 
 
 @dataclasses.dataclass
@@ -87,8 +90,8 @@ class LLaMAConfig(ModelConfig):
             problems.append(f"head size {self.emb_dim // self.nheads} is odd: rotary pairs need an even size")
         if self.kvheads < 0 or (self.kvheads and self.nheads % self.kvheads):
             problems.append(f"nheads {self.nheads} is not a multiple of kvheads {self.kvheads}")
-        if self.activation_fn not in ("swish", "silu"):
-            problems.append(f"activation_fn {self.activation_fn!r}: Llama's feed-forward gates with swish/silu")
+        if str(self.activation_fn).lower() not in ACTIVATION_NAMES:
+            problems.append(f"activation_fn {self.activation_fn!r} is not one of {', '.join(ACTIVATION_NAMES)}")
         if self.p_dropout:
             problems.append("p_dropout must be 0: this library only generates")
         kind = (self.rope_scaling or {}).get("rope_type", "regular")
@@ -135,9 +138,9 @@ class LLaMAConfig(ModelConfig):
                 f"config.json head_dim {hf['head_dim']} differs from hidden_size/num_attention_heads "
                 f"{width}/{heads}: the reference's Llama fixes the head size to that quotient"
             )
-        act = hf.get("hidden_act", "silu")
-        if act not in ("silu", "swish"):
-            raise ValueError(f"config.json hidden_act {act!r}: Llama's feed-forward gates with silu")
+        act = str(hf.get("hidden_act", "silu")).lower()
+        if act not in ACTIVATION_NAMES:
+            raise ValueError(f"config.json hidden_act {act!r} is not one of {', '.join(ACTIVATION_NAMES)}")
         kv = hf.get("num_key_value_heads")
         kwargs = dict(
             src_vocab_size=hf["vocab_size"],
@@ -153,6 +156,7 @@ class LLaMAConfig(ModelConfig):
             tie_heads=bool(hf.get("tie_word_embeddings", False)),
             attn_bias=bool(hf.get("attention_bias", False)),
             mlp_bias=bool(hf.get("mlp_bias", False)),
+            activation_fn="swish" if act == "silu" else act,
         )
         if rope_theta is not None:
             kwargs["rope_theta"] = float(rope_theta)
@@ -178,7 +182,7 @@ class LLaMAConfig(ModelConfig):
             "tie_word_embeddings": self.tie_heads,
             "attention_bias": self.attn_bias,
             "mlp_bias": self.mlp_bias,
-            "hidden_act": "silu",
+            "hidden_act": "silu" if str(self.activation_fn).lower() in ("swish", "silu") else str(self.activation_fn).lower(),
             "head_dim": self.head_dim,
         }
         return out

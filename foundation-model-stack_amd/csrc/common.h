@@ -62,6 +62,30 @@ __device__ __forceinline__ bf16 from_f32<bf16>(float x) {
 }
 
 // --------------------------------------------------------------------------
+// activation functions (the codes are FMS_ACT_* of fmsamd.h), in float32
+// --------------------------------------------------------------------------
+__device__ __forceinline__ float fms_activate(float x, int kind) {
+  switch (kind) {
+    case 0:  // silu
+      return x / (1.f + expf(-x));
+    case 1:  // gelu
+      return 0.5f * x * (1.f + erff(x * 0.70710678118654752f));
+    case 2:  // relu
+      return fmaxf(x, 0.f);
+    case 4:  // sigmoid
+      return 1.f / (1.f + expf(-x));
+    case 5:  // tanh
+      return tanhf(x);
+    case 6:  // mish; log(1 + e^x) is x itself beyond 20, as the reference's library has it
+      return x * tanhf(x > 20.f ? x : log1pf(expf(x)));
+    case 7:  // gelu, tanh approximation
+      return 0.5f * x * (1.f + tanhf(0.79788456080286536f * (x + 0.044715f * x * x * x)));
+    default:  // identity
+      return x;
+  }
+}
+
+// --------------------------------------------------------------------------
 // reductions
 // --------------------------------------------------------------------------
 __device__ __forceinline__ float wave_sum(float v) {

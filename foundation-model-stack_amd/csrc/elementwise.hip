@@ -247,18 +247,7 @@ extern "C" int fmsamd_add_norm(float* resid, const void* branch, int act_dtype, 
 // --------------------------------------------------------------------------
 // gated activation: out[t, j] = act(gu[t, j] + bg[j]) * (gu[t, hidden + j] + bu[j])
 // --------------------------------------------------------------------------
-__device__ __forceinline__ float activate(float x, int kind) {
-  switch (kind) {
-    case FMS_ACT_SILU:
-      return x / (1.f + expf(-x));
-    case FMS_ACT_GELU:
-      return 0.5f * x * (1.f + erff(x * 0.70710678118654752f));
-    case FMS_ACT_RELU:
-      return fmaxf(x, 0.f);
-    default:
-      return x;
-  }
-}
+__device__ __forceinline__ float activate(float x, int kind) { return fms_activate(x, kind); }
 
 // VEC elements per thread and step: 16 bytes of the activation type when the row length allows it
 template <int VEC, typename T, typename BiasT>
@@ -313,7 +302,7 @@ extern "C" int fmsamd_gated_act(const void* gu, const void* bias, int bias_dtype
                                 int hidden, int act, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   FMS_REQUIRE(n_tokens > 0 && hidden > 0, "gated_act: bad sizes T=%d hidden=%d", n_tokens, hidden);
-  FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gated_act: unknown activation %d", act);
+  FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_LAST, "gated_act: unknown activation %d", act);
   FMS_REQUIRE(n_tokens <= 65535, "gated_act: %d tokens exceed one launch (65535)", n_tokens);
   if (dtype == FMS_F32 && (bias == nullptr || bias_dtype == FMS_F32))
     launch_gated_act<float, float>(gu, bias, out, n_tokens, hidden, act, stream);

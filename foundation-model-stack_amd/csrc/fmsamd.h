@@ -14,9 +14,14 @@
 
 // activations of the gated feed-forward
 #define FMS_ACT_SILU 0
-#define FMS_ACT_GELU 1
+#define FMS_ACT_GELU 1       // with the error function
 #define FMS_ACT_RELU 2
 #define FMS_ACT_IDENTITY 3
+#define FMS_ACT_SIGMOID 4
+#define FMS_ACT_TANH 5
+#define FMS_ACT_MISH 6       // x tanh(log(1 + e^x))
+#define FMS_ACT_GELU_TANH 7  // the tanh approximation
+#define FMS_ACT_LAST FMS_ACT_GELU_TANH
 
 #ifdef __cplusplus
 extern "C" {

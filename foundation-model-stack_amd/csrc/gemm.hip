@@ -637,7 +637,7 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
               ldx);
   FMS_REQUIRE(ldx >= K && ldo >= hidden, "gemm_skinny_gated_bf16: leading dimensions too small");
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_gated_bf16: unknown output dtype %d", out_dtype);
-  FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_IDENTITY, "gemm_skinny_gated_bf16: unknown activation %d", act);
+  FMS_REQUIRE(act >= FMS_ACT_SILU && act <= FMS_ACT_LAST, "gemm_skinny_gated_bf16: unknown activation %d", act);
   if (M > 16)
     return wide_product(EPI_GATED, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, hidden, K, hidden, act, scale,
                         RopeEpilogue{}, ResidEpilogue{}, workspace, workspace_bytes, stream);

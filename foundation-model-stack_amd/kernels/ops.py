@@ -18,7 +18,9 @@ import torch
 from .library import check, load
 
 F32, BF16 = 0, 1
-ACTIVATIONS = {"silu": 0, "swish": 0, "gelu": 1, "relu": 2, "identity": 3}
+# the names of the reference (fms/utils/activation.py:14-24) and "identity"; the numbers are FMS_ACT_* of csrc/fmsamd.h
+ACTIVATIONS = {"silu": 0, "swish": 0, "gelu": 1, "relu": 2, "identity": 3, "sigmoid": 4, "tanh": 5, "mish": 6,
+               "gelu-tanh": 7, "gelu_pytorch_tanh": 7}
 PAGE_TOKENS = 64
 
 

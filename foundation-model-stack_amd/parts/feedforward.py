@@ -17,6 +17,7 @@ from .linear import Linear
 class GatedLinearUnit(FeedForward):
     def __init__(self, width: int, hidden_dim: int, activation: str = "swish", use_bias: bool = False):
         super().__init__()
+        activation = str(activation).lower()  # the reference looks names up without regard to case
         if activation not in ops.ACTIVATIONS:
             raise ValueError(f"activation {activation!r} is not one of {sorted(ops.ACTIVATIONS)}")
         self.width, self.hidden_dim, self.activation = width, int(hidden_dim), activation

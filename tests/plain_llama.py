@@ -39,6 +39,7 @@ class PlainConfig:
     attn_bias: bool = False
     mlp_bias: bool = False
     rope_scaling: dict = field(default_factory=dict)
+    activation: str = "swish"  # activation_fn (fms/models/llama.py:51)
 
     @property
     def head_dim(self) -> int:
@@ -169,6 +170,23 @@ def silu(x: torch.Tensor) -> torch.Tensor:
     return x * torch.sigmoid(x)
 
 
+def activation(name: str):
+    """fms/utils/activation.py:14-24, 47-50: the activation functions by name (case ignored); "gelu" is the one
+    with the error function, the two "gelu...tanh" names its tanh approximation."""
+    table = {
+        "swish": silu,
+        "silu": silu,
+        "gelu": lambda x: 0.5 * x * (1.0 + torch.erf(x / math.sqrt(2.0))),
+        "gelu-tanh": lambda x: 0.5 * x * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (x + 0.044715 * x**3))),
+        "mish": lambda x: x * torch.tanh(torch.nn.functional.softplus(x)),
+        "relu": lambda x: torch.clamp(x, min=0.0),
+        "sigmoid": torch.sigmoid,
+        "tanh": torch.tanh,
+    }
+    table["gelu_pytorch_tanh"] = table["gelu-tanh"]
+    return table[name.lower()]
+
+
 def gated_feed_forward(
     x: torch.Tensor,
     wg1_fused: torch.Tensor,
@@ -177,6 +195,7 @@ def gated_feed_forward(
     bias2: Optional[torch.Tensor] = None,
     storage=None,
     rounding: str = "stored",
+    act_name: str = "swish",
 ) -> torch.Tensor:
     """fms/modules/feedforward.py:288-297: first half of the fused rows is the gate.
 
@@ -186,7 +205,8 @@ def gated_feed_forward(
     hidden = wg1_fused.shape[0] // 2
     both = st(linear(x, wg1_fused, bias_fused))
     gate, up = both[..., :hidden], both[..., hidden:]
-    act = st(silu(gate)) if rounding == "reference" else silu(gate)
+    fn = activation(act_name)
+    act = st(fn(gate)) if rounding == "reference" else fn(gate)
     return linear(st(act * up), w2, bias2)
 
 
@@ -308,6 +328,7 @@ def forward(
             w.get(p + "ff_sub_layer.w2.bias"),
             storage,
             rounding,
+            cfg.activation,
         ))
         x = rs(h + residual)
     x = norm(x, w["base_model.dec_norm.weight"])
@@ -424,6 +445,9 @@ def config_from_hf(cfg: dict) -> PlainConfig:
         attn_bias=bool(cfg.get("attention_bias", False)),
         mlp_bias=bool(cfg.get("mlp_bias", False)),
         rope_scaling=rope_scaling or {},
+        # the reference's builder does not read hidden_act (its models keep activation_fn's default); a folder that
+        # names another function is run with that one here
+        activation=cfg.get("hidden_act", "silu"),
     )
 
 

@@ -37,9 +37,9 @@ CONFIGS = {
     # head size 64 with grouped kv heads (the MFMA kernels' other compile-time head size), a larger vocabulary
     "E": dict(src_vocab_size=1000, emb_dim=256, nheads=4, kvheads=2, nlayers=2, hidden_dim=344, multiple_of=1,
               norm_eps=1e-5, rope_theta=500000.0, max_expected_seq_len=512, tie_heads=True),
-    # head size 96 (a multiple of 16 that no kernel is specialised for), one kv head
+    # head size 96 (a multiple of 16 that no kernel is specialised for), one kv head, another activation function
     "F": dict(src_vocab_size=333, emb_dim=192, nheads=2, kvheads=1, nlayers=1, hidden_dim=520, multiple_of=1,
-              norm_eps=1e-6, rope_theta=10000.0, max_expected_seq_len=512, tie_heads=False),
+              norm_eps=1e-6, rope_theta=10000.0, max_expected_seq_len=512, tie_heads=False, activation_fn="gelu-tanh"),
 }
 DTYPES = ["float32", "bfloat16"]
 

@@ -50,7 +50,7 @@ def test_config_round_trip_and_updated(tmp_path):
 
 
 @pytest.mark.parametrize("bad", [dict(emb_dim=100, nheads=3), dict(nheads=4, kvheads=3), dict(emb_dim=12, nheads=4),
-                                 dict(activation_fn="gelu"), dict(rope_scaling={"rope_type": "yarn"})])
+                                 dict(activation_fn="gelu_new"), dict(rope_scaling={"rope_type": "yarn"})])
 def test_config_refuses_impossible_numbers(bad):
     with pytest.raises(ValueError):
         LLaMAConfig(**bad)
@@ -79,8 +79,12 @@ def test_config_from_hugging_face_keys():
     assert c.rope_theta == 5e5 and c.rope_scaling["rope_type"] == "llama3"
     with pytest.raises(ValueError):
         LLaMAConfig.from_hf_dict(dict(hf, head_dim=16))
+    # hidden_act, which the reference's builder does not read, becomes activation_fn: one of the names that the
+    # reference's activation table has (fms/utils/activation.py:14-24)
+    assert c.activation_fn == "swish" and LLaMAConfig.from_hf_dict(dict(hf, hidden_act="gelu")).activation_fn == "gelu"
+    assert LLaMAConfig.from_hf_dict(LLaMAConfig(emb_dim=64, nheads=4, activation_fn="Mish").to_hf_dict()).activation_fn == "mish"
     with pytest.raises(ValueError):
-        LLaMAConfig.from_hf_dict(dict(hf, hidden_act="gelu"))
+        LLaMAConfig.from_hf_dict(dict(hf, hidden_act="gelu_new"))
     with pytest.raises(ValueError):
         LLaMAConfig.from_hf_dict({k: v for k, v in hf.items() if k != "vocab_size"})
 

@@ -91,15 +91,19 @@ def test_rotary_part(lib):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows", [3, 100])
-def test_feed_forward_part(lib, dtype, rows):
+@pytest.mark.parametrize("rows,activation", [(3, "swish"), (100, "swish"), (3, "gelu"), (40, "gelu-tanh"), (100, "mish"), (9, "relu"),
+                                             (20, "sigmoid"), (100, "tanh"), (3, "GELU_pytorch_tanh")])
+def test_feed_forward_part(lib, dtype, rows, activation):
+    """Every activation function the reference knows by name (fms/utils/activation.py:14-24), at row counts that
+    take the products for few rows (gate and activation inside the product) and the separate activation kernel."""
     from fms_amd.parts import make_part
 
-    ff = make_part("feed_forward", "glu", width=40, hidden_dim=72, activation="swish", use_bias=True)
+    ff = make_part("feed_forward", "glu", width=40, hidden_dim=72, activation=activation, use_bias=True)
     w = bind_random(ff, dtype, seed=1)
     x = torch.randn(rows, 40).to(dtype)
     out = ff.forward(x.to(DEV)).cpu().float()
-    want = P.gated_feed_forward(x.float(), w["wg1_fused.weight"], w["w2.weight"], w["wg1_fused.bias"], w["w2.bias"])
+    want = P.gated_feed_forward(x.float(), w["wg1_fused.weight"], w["w2.weight"], w["wg1_fused.bias"], w["w2.bias"],
+                                act_name=activation)
     torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=0.1, rtol=5e-2)))
 
 
