@@ -241,6 +241,38 @@ def reference_attention(qs, ks, vs, starts, H, K, scale=None, window=0):
     return torch.cat(outs).reshape(sum(q.shape[0] for q in qs), -1)
 
 
+def reference_attention_rows(qs, ks, vs, starts, H, K, scale=None, window=0):
+    """The same attention for the query rows only (fms/modules/attention.py:215-294: head h reads kv head
+    h // (H / K), key j is visible to the query at position p if j <= p, and p - j < window if there is one):
+    for contexts so long that the whole square of scores of causal_attention would not fit."""
+    outs = []
+    for q, k, v, s in zip(qs, ks, vs, starts):
+        n, _, D = q.shape
+        sc = scale if scale is not None else 1 / math.sqrt(D)
+        pos = torch.arange(s, s + n)[:, None]
+        key = torch.arange(k.shape[0])[None, :]
+        visible = key <= pos
+        if window:
+            visible &= pos - key < window
+        o = torch.zeros(n, H, D)
+        for h in range(H):
+            kh = h // (H // K)
+            scores = (q[:, h].double() @ k[:, kh].double().t()) * sc
+            probs = torch.softmax(scores.masked_fill(~visible, float("-inf")), dim=-1)
+            o[:, h] = (probs @ v[:, kh].double()).float()
+        outs.append(o)
+    return torch.cat(outs).reshape(sum(q.shape[0] for q in qs), -1)
+
+
+def test_the_two_attention_references_agree():
+    torch.manual_seed(3)
+    ks, vs = [torch.randn(90, 2, 16)], [torch.randn(90, 2, 16)]
+    qs = [torch.randn(7, 4, 16)]
+    for window in (0, 20):
+        torch.testing.assert_close(reference_attention_rows(qs, ks, vs, [83], 4, 2, window=window),
+                                   reference_attention(qs, ks, vs, [83], 4, 2, window=window), atol=1e-5, rtol=1e-5)
+
+
 def attention_case(ops, dtype, H, K, D, starts, lens, window=0, decode=False, scale=None, spike=False, **kw):
     torch.manual_seed(5)
     totals = [s + n for s, n in zip(starts, lens)]
@@ -277,7 +309,8 @@ def attention_case(ops, dtype, H, K, D, starts, lens, window=0, decode=False, sc
         decode=decode, max_context=max(totals),
         qblock_start=dev(torch.tensor(qb_start, dtype=torch.int32)), qblock_len=dev(torch.tensor(qb_len, dtype=torch.int32)), qblock_tokens=qblock, **kw,
     )
-    want = reference_attention(qs, ks, vs, starts, H, K, scale=sc, window=window)
+    rows_only = max(totals) > 3000  # the whole square of scores of a long context is too much for the plain function
+    want = (reference_attention_rows if rows_only else reference_attention)(qs, ks, vs, starts, H, K, scale=sc, window=window)
     torch.testing.assert_close(out.cpu().float(), want, **(dict(atol=3e-5, rtol=3e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)))
 
 
@@ -322,6 +355,24 @@ def test_attention_far_key_and_window(ops, dtype, decode):
     attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=100)
     attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=64, scale=0.3)
     attention_case(ops, dtype, 4, 2, 32, starts=[900, 130], lens=lens, decode=decode, window=1)
+
+
+def test_attention_over_long_contexts(ops):
+    """Contexts of 8200, 12000 and 20000 tokens beside short ones: the decode kernel with the split that the wrapper
+    picks for such a bound and with others, pages through LDS and not, a far key that decides the result, a window
+    whose edge lies thousands of tokens back; the prefill kernel for a chunk behind a cached prefix of 8000 tokens;
+    the float32 kernel."""
+    bf, f32 = torch.bfloat16, torch.float32
+    attention_case(ops, bf, 8, 2, 128, starts=[8199, 19999, 2], lens=[1, 1, 1], decode=True, spike=True)
+    attention_case(ops, bf, 8, 2, 128, starts=[8199, 19999, 2, 700], lens=[1, 1, 1, 1], decode=True, staged=True)
+    attention_case(ops, bf, 8, 2, 128, starts=[8199, 19999, 2], lens=[1, 1, 1], decode=True, staged=True, window=5000)
+    attention_case(ops, bf, 8, 2, 128, starts=[19999, 64], lens=[1, 1], decode=True, staged=True, pages_per_block=40, waves=8, spike=True)
+    attention_case(ops, bf, 4, 1, 64, starts=[11999, 0], lens=[1, 1], decode=True, spike=True)
+    attention_case(ops, bf, 6, 2, 80, starts=[9000], lens=[1], decode=True, window=4097)
+    attention_case(ops, bf, 8, 2, 128, starts=[8000, 0], lens=[200, 70], spike=True)
+    attention_case(ops, bf, 4, 4, 32, starts=[5000], lens=[100], window=3000)
+    attention_case(ops, f32, 4, 2, 16, starts=[9000, 5], lens=[3, 2], spike=True)
+    attention_case(ops, f32, 4, 2, 16, starts=[9000], lens=[1], decode=True)
 
 
 def test_attention_generic_bf16_agrees(ops):
