@@ -360,7 +360,7 @@ def test_attention_far_key_and_window(ops, dtype, decode):
 def test_attention_over_long_contexts(ops):
     """Contexts of 8200, 12000 and 20000 tokens beside short ones: the decode kernel with the split that the wrapper
     picks for such a bound and with others, pages through LDS and not, a far key that decides the result, a window
-    whose edge lies thousands of tokens back; the prefill kernel for a chunk behind a cached prefix of 8000 tokens;
+    whose edge lies thousands of tokens back; the prefill kernel for a chunk behind a cached prefix of 8000 tokens and for a prompt of 3200 tokens;
     the float32 kernel."""
     bf, f32 = torch.bfloat16, torch.float32
     attention_case(ops, bf, 8, 2, 128, starts=[8199, 19999, 2], lens=[1, 1, 1], decode=True, spike=True)
@@ -370,6 +370,7 @@ def test_attention_over_long_contexts(ops):
     attention_case(ops, bf, 4, 1, 64, starts=[11999, 0], lens=[1, 1], decode=True, spike=True)
     attention_case(ops, bf, 6, 2, 80, starts=[9000], lens=[1], decode=True, window=4097)
     attention_case(ops, bf, 8, 2, 128, starts=[8000, 0], lens=[200, 70], spike=True)
+    attention_case(ops, bf, 8, 2, 128, starts=[0, 0], lens=[3200, 33], spike=True)  # a long prompt whole: a hundred query blocks
     attention_case(ops, bf, 4, 4, 32, starts=[5000], lens=[100], window=3000)
     attention_case(ops, f32, 4, 2, 16, starts=[9000, 5], lens=[3, 2], spike=True)
     attention_case(ops, f32, 4, 2, 16, starts=[9000], lens=[1], decode=True)
