@@ -527,6 +527,25 @@ def test_qkv_rope_write_takes_a_deferred_row_norm(ops):
         torch.testing.assert_close(a, b, atol=0.02 * float(a.abs().max()), rtol=2e-2)
 
 
+@pytest.mark.parametrize("vocab,width", [(128256, 4096), (32000, 4096), (49152, 2560)])
+def test_output_head_at_served_vocabularies(ops, vocab, width):
+    """The last product of a step at the vocabularies and widths of the registered variants: float32 logits from
+    bfloat16 rows, for the row counts of decode batches (the weight-streaming kernels, 1 to 128 rows, in blocks of
+    thousands) and above (this package's MFMA kernel), against the float32 product of the same operands; and the
+    token choice on those logits."""
+    torch.manual_seed(21)
+    w = (torch.randn(vocab, width, device="cuda") * 0.02).bfloat16()
+    wf = w.float()
+    for M in (1, 8, 17, 33, 64, 128, 130):
+        x = torch.randn(M, width, device="cuda").bfloat16()
+        got = ops.linear(x, w, None, out_dtype=torch.float32)
+        want = x.float() @ wf.t()
+        assert got.dtype == torch.float32 and tuple(got.shape) == (M, vocab)
+        torch.testing.assert_close(got, want, atol=2e-3, rtol=2e-3)
+        assert ops.sample(got, False).tolist() == got.argmax(-1).tolist()
+    del wf
+
+
 # --------------------------------------------------------------------------
 def test_argmax(ops):
     torch.manual_seed(9)
