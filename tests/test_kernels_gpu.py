@@ -500,6 +500,62 @@ def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
             torch.testing.assert_close(stream2.cpu(), resid + normed @ w2.float().t(), **bound)
 
 
+@pytest.mark.parametrize("E,F,H,K", [(5120, 13824, 40, 40), (8192, 28672, 64, 8), (2560, 10240, 32, 32)])
+def test_decode_products_at_the_layer_sizes_of_other_variants(ops, E, F, H, K):
+    """The four products of a layer as a decode step runs them, at the sizes of the 13B, 70B and granite 3B variants
+    (the 8B and 7B sizes run through whole models in test_model_shapes_gpu.py): output projection into the stream,
+    gate/up with the activation and the deferred norm, down projection into the stream, qkv with rotation and cache
+    write and the deferred norm.  Row counts of the kernels for up to 16 rows, for 17 to 32 and for 33 to 128.
+    References are float32 products of the same operands, on the GPU."""
+    torch.manual_seed(31)
+    D = E // H
+    eps = 1e-5
+    wo = (torch.randn(E, E, device="cuda") * 0.02).bfloat16()
+    wgu = (torch.randn(2 * F, E, device="cuda") * 0.02).bfloat16()
+    wd = (torch.randn(E, F, device="cuda") * 0.02).bfloat16()
+    wqkv = (torch.randn((H + 2 * K) * D, E, device="cuda") * 0.02).bfloat16()
+    nw = (1 + 0.1 * torch.randn(E, device="cuda")).bfloat16()
+    cos, sin = ops.rope_table(dev(P.rope_frequencies(D, 10000.0)), 512)
+    for M in (8, 24, 80):
+        attn = torch.randn(M, E, device="cuda").bfloat16()
+        resid = torch.randn(M, E, device="cuda") * 2
+        resid[0] *= 20
+        stream = resid.clone()
+        # output projection: stream += attn Wo^T, scaled = stream * norm weight, partial sums of squares
+        scaled, row_norm = ops.linear_into_stream(attn, wo, None, stream, nw, eps)
+        want_stream = resid + attn.float() @ wo.float().t()
+        torch.testing.assert_close(stream, want_stream, atol=2e-3, rtol=1e-4)
+        normed = want_stream * torch.rsqrt(want_stream.pow(2).mean(-1, keepdim=True) + eps) * nw.float()
+        # gate/up with the deferred norm
+        hidden = ops.gated_linear(scaled, wgu, None, "swish", row_norm=row_norm)
+        gu = normed @ wgu.float().t()
+        want_hidden = P.silu(gu[:, :F]) * gu[:, F:]
+        torch.testing.assert_close(hidden.float(), want_hidden, atol=0.02 * float(want_hidden.abs().max()) + 1e-3, rtol=2e-2)
+        # down projection into the stream
+        stream2 = want_stream.clone()
+        ops.linear_into_stream(hidden, wd, None, stream2, nw, eps)
+        torch.testing.assert_close(stream2, want_stream + hidden.float() @ wd.float().t(), atol=3e-3, rtol=1e-4)
+        # qkv with rotation and cache write, against the product followed by the separate rotation kernel
+        positions = torch.randint(0, 300, (M,)).int()
+        seq = torch.arange(M).int()
+        table, n_pages = make_pages([320] * M, K, D, torch.bfloat16, seed=4)
+        res = []
+        for fused in (True, False):
+            kc = torch.zeros(n_pages, K, PAGE, D, dtype=torch.bfloat16, device="cuda")
+            vc = torch.zeros(n_pages, K, D, PAGE, dtype=torch.bfloat16, device="cuda")
+            args = (dev(positions), dev(seq), dev(table), cos, sin, D, kc, vc, H, K, D)
+            if fused:
+                qkv = ops.qkv_rope_write(scaled, wqkv, None, *args, row_norm=row_norm)
+            else:
+                qkv = (normed @ wqkv.float().t()).bfloat16()
+                ops.rope_kv_write(qkv, *args)
+            res.append((qkv[:, : H * D].float(), kc.float(), vc.float()))
+        step = 2.0 ** -7 * max(float(res[1][0].abs().max()), float(res[1][1].abs().max()))  # see test_qkv_rope_write
+        for a, b in zip(res[0], res[1]):
+            assert float(b.abs().max()) > 0
+            torch.testing.assert_close(a, b, atol=step, rtol=2e-2)
+
+
 def test_qkv_rope_write_takes_a_deferred_row_norm(ops):
     torch.manual_seed(13)
     M, H, K, D, E, eps = 5, 4, 2, 32, 96, 1e-5
