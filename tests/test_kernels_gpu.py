@@ -320,7 +320,8 @@ def test_attention_generic_f32(ops, H, K, D):
     attention_case(ops, torch.float32, H, K, D, starts=[299, 64], lens=[1, 1], decode=True)
 
 
-@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (6, 3, 128), (2, 2, 64), (32, 1, 32), (2, 1, 256), (5, 5, 80), (8, 2, 128), (12, 2, 64)])
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (6, 3, 128), (2, 2, 64), (32, 1, 32), (2, 1, 256), (5, 5, 80), (8, 2, 128), (12, 2, 64),
+                                   (16, 2, 128), (4, 4, 128), (24, 1, 128)])
 def test_attention_prefill_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 0, 0], lens=[200, 1, 33])
     # a chunk that continues a cached prefix
@@ -328,7 +329,8 @@ def test_attention_prefill_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 30], lens=[300, 100])
 
 
-@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (8, 2, 128), (2, 2, 64), (40, 2, 32), (2, 1, 256), (5, 5, 80)])
+@pytest.mark.parametrize("H,K,D", [(4, 2, 16), (4, 1, 48), (8, 2, 128), (2, 2, 64), (40, 2, 32), (2, 1, 256), (5, 5, 80),
+                                   (16, 2, 128), (4, 4, 128), (24, 1, 128)])
 def test_attention_decode_bf16(ops, H, K, D):
     attention_case(ops, torch.bfloat16, H, K, D, starts=[0, 63, 64, 700], lens=[1, 1, 1, 1], decode=True)
     attention_case(ops, torch.bfloat16, H, K, D, starts=[1500, 2], lens=[1, 1], decode=True, pages_per_block=2, waves=1)
