@@ -90,15 +90,17 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, long row_stride, const
 }
 
 // The same for many tokens: a block takes RT consecutive token rows and one head (a query head, a key head or
-// a value head), four elements a thread.  Rows of q and k stay rows; the values of a head are turned over in
-// LDS, so that the lanes of a store are neighbouring tokens of one row of the transposed page (tokens that
-// follow one another in a sequence are neighbours there) instead of 2-byte writes 128 bytes apart.
-template <typename T>
-struct Vec4 {
-  typedef T type __attribute__((ext_vector_type(4)));
+// a value head), 16 bytes a thread and step where rows allow it (QV = 8 bfloat16 or 4 float32 elements, with
+// their cosines and sines as 16-byte loads too; QV = 4 for bfloat16 rows that only allow 8 bytes).  Rows of q and
+// k stay rows; the values of a head are turned over in LDS, so that the lanes of a store are neighbouring tokens
+// of one row of the transposed page (tokens that follow one another in a sequence are neighbours there) instead
+// of 2-byte writes 128 bytes apart.
+template <typename T, int N>
+struct VecOf {
+  typedef T type __attribute__((ext_vector_type(N)));
 };
 
-template <typename T>
+template <typename T, int QV>
 __global__ void __launch_bounds__(256)
     rope_kv_tile_kernel(T* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
                         const int* __restrict__ seq_of_token, const int* __restrict__ block_table, int table_stride,
@@ -106,7 +108,8 @@ __global__ void __launch_bounds__(256)
                         T* __restrict__ k_cache, T* __restrict__ v_cache, int nheads, int kvheads, int head_dim,
                         int n_tokens) {
   constexpr int RT = sizeof(T) == 4 ? 32 : 64;
-  typedef typename Vec4<T>::type vec4;
+  typedef typename VecOf<T, 4>::type vec4;
+  typedef typename VecOf<T, QV>::type vecq;
   extern __shared__ __attribute__((aligned(16))) unsigned char tile_raw[];  // value heads: RT x (head_dim + 4)
   __shared__ int s_pos[RT];
   __shared__ long long s_page[RT];  // -1: the row is padding or past the end
@@ -133,32 +136,45 @@ __global__ void __launch_bounds__(256)
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
 
   if (hh < nheads + kvheads) {
-    for (int idx = threadIdx.x; idx < RT * quads; idx += blockDim.x) {
-      const int tok = idx / quads, qd = idx - tok * quads;
+    const int per_row = head_dim / QV;  // the host has checked that QV divides the head size
+    for (int idx = threadIdx.x; idx < RT * per_row; idx += blockDim.x) {
+      const int tok = idx / per_row, qd = idx - tok * per_row;
       if (s_page[tok] < 0) continue;
       const int pos = s_pos[tok];
-      T* p = qkv + (size_t)(t0 + tok) * row_stride + (size_t)hh * head_dim + 4 * qd;
-      vec4 v = *reinterpret_cast<const vec4*>(p);
+      T* p = qkv + (size_t)(t0 + tok) * row_stride + (size_t)hh * head_dim + QV * qd;
+      vecq v = *reinterpret_cast<const vecq*>(p);
       if (cos_t != nullptr) {
         const int tpos = pos < 0 ? 0 : (pos < max_pos ? pos : max_pos - 1);  // the host has checked; never read outside the table
+        const int i0 = (QV / 2) * qd;  // the first pair (x[2i], x[2i+1]) of this piece
+        float c[QV / 2], sn[QV / 2];
+        if (QV == 8 && i0 + 4 <= rot_half && rot_half % 4 == 0) {  // four angles: 16 bytes each of cosines and sines
+          const f32x4 c4 = *reinterpret_cast<const f32x4*>(cos_t + (size_t)tpos * rot_half + i0);
+          const f32x4 s4 = *reinterpret_cast<const f32x4*>(sin_t + (size_t)tpos * rot_half + i0);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int i = 2 * qd + j;  // the pair (x[2i], x[2i+1])
-          if (i < rot_half) {
-            const float c = cos_t[(size_t)tpos * rot_half + i];
-            const float sn = sin_t[(size_t)tpos * rot_half + i];
+          for (int j = 0; j < QV / 2; ++j) c[j] = c4[j & 3], sn[j] = s4[j & 3];
+        } else {
+#pragma unroll
+          for (int j = 0; j < QV / 2; ++j) {
+            const bool rotates = i0 + j < rot_half;
+            c[j] = rotates ? cos_t[(size_t)tpos * rot_half + i0 + j] : 1.f;
+            sn[j] = rotates ? sin_t[(size_t)tpos * rot_half + i0 + j] : 0.f;
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < QV / 2; ++j) {
+          if (i0 + j < rot_half) {
             const float a = to_f32(v[2 * j]), b = to_f32(v[2 * j + 1]);
-            v[2 * j] = from_f32<T>(c * a - sn * b);
-            v[2 * j + 1] = from_f32<T>(sn * a + c * b);
+            v[2 * j] = from_f32<T>(c[j] * a - sn[j] * b);
+            v[2 * j + 1] = from_f32<T>(sn[j] * a + c[j] * b);
           }
         }
       }
       if (hh < nheads) {
-        *reinterpret_cast<vec4*>(p) = v;
+        *reinterpret_cast<vecq*>(p) = v;
       } else {
         const int kh = hh - nheads;
-        T* dst = k_cache + (size_t)s_page[tok] * page_elems + ((size_t)kh * PAGE_TOKENS + pos % PAGE_TOKENS) * head_dim + 4 * qd;
-        *reinterpret_cast<vec4*>(dst) = v;
+        T* dst = k_cache + (size_t)s_page[tok] * page_elems + ((size_t)kh * PAGE_TOKENS + pos % PAGE_TOKENS) * head_dim + QV * qd;
+        *reinterpret_cast<vecq*>(dst) = v;
       }
     }
     return;
@@ -172,8 +188,43 @@ __global__ void __launch_bounds__(256)
     *reinterpret_cast<vec4*>(tile + tok * ld + 4 * qd) =
         *reinterpret_cast<const vec4*>(qkv + (size_t)(t0 + tok) * row_stride + (size_t)hh * head_dim + 4 * qd);
   }
+  // TG tokens make 16 bytes of a row of the transposed page.  Where the TG tokens of a group follow one another
+  // in one page, from a place that is a multiple of TG (a prompt's tokens do), they leave as one 16-byte store,
+  // and the lanes of a wave fill whole rows of the page; other groups go element by element.
+  constexpr int TG = (QV == 8 || sizeof(T) == 4) ? 16 / (int)sizeof(T) : 1;
+  __shared__ int s_together[RT];
+  if (TG > 1 && threadIdx.x < RT / TG) {
+    const int tok0 = threadIdx.x * TG;
+    bool together = s_page[tok0] >= 0 && (s_pos[tok0] % PAGE_TOKENS) % TG == 0;
+    for (int j = 1; j < TG; ++j) together = together && s_page[tok0 + j] == s_page[tok0] && s_pos[tok0 + j] == s_pos[tok0] + j;
+    s_together[threadIdx.x] = together ? 1 : 0;
+  }
   __syncthreads();
   const int kh = hh - nheads - kvheads;
+  if constexpr (TG > 1) {
+    typedef typename VecOf<T, TG>::type vecg;
+    constexpr int GROUPS = RT / TG;
+    for (int idx = threadIdx.x; idx < GROUPS * head_dim; idx += blockDim.x) {
+      const int tg = idx % GROUPS, d = idx / GROUPS;  // neighbouring lanes: neighbouring pieces of a row
+      const int tok0 = tg * TG;
+      if (s_together[tg]) {
+        vecg v;
+#pragma unroll
+        for (int j = 0; j < TG; ++j) v[j] = tile[(tok0 + j) * ld + d];
+        *reinterpret_cast<vecg*>(v_cache + (size_t)s_page[tok0] * page_elems + ((size_t)kh * head_dim + d) * PAGE_TOKENS +
+                                 s_pos[tok0] % PAGE_TOKENS) = v;
+      } else {
+#pragma unroll
+        for (int j = 0; j < TG; ++j) {
+          const int tok = tok0 + j;
+          if (s_page[tok] >= 0)
+            v_cache[(size_t)s_page[tok] * page_elems + ((size_t)kh * head_dim + d) * PAGE_TOKENS + s_pos[tok] % PAGE_TOKENS] =
+                tile[tok * ld + d];
+        }
+      }
+    }
+    return;
+  }
   for (int idx = threadIdx.x; idx < RT * head_dim; idx += blockDim.x) {
     const int tok = idx % RT, d = idx / RT;  // neighbouring lanes: neighbouring tokens
     if (s_page[tok] < 0) continue;
@@ -200,18 +251,26 @@ extern "C" int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const
   FMS_REQUIRE(dtype == FMS_F32 || dtype == FMS_BF16, "rope_kv_write: unknown dtype %d", dtype);
   // four elements a thread need rows that start at multiples of four elements
   const bool by_fours = head_dim % 4 == 0 && row_stride % 4 == 0 && (uintptr_t)qkv % (4 * elem) == 0 &&
-                        (uintptr_t)k_cache % (4 * elem) == 0;
+                        (uintptr_t)k_cache % (4 * elem) == 0 && (uintptr_t)v_cache % (4 * elem) == 0;
   if (by_fours) {
     const int rt = dtype == FMS_F32 ? 32 : 64;
     FMS_REQUIRE(nheads + 2 * kvheads <= 65535, "rope_kv_write: too many heads");
     dim3 grid(ceil_div(n_tokens, rt), nheads + 2 * kvheads);
     const size_t lds = (size_t)rt * (head_dim + 4) * elem;
+    // bfloat16 rows of q and k by eights (16 bytes) where heads, rows, tables and caches start at multiples of 16 bytes
+    const bool by_eights = dtype == FMS_BF16 && head_dim % 8 == 0 && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0 &&
+                           (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0 && (uintptr_t)cos_t % 16 == 0 &&
+                           (uintptr_t)sin_t % 16 == 0;
     if (dtype == FMS_F32)
-      rope_kv_tile_kernel<float><<<grid, threads, lds, stream>>>(
+      rope_kv_tile_kernel<float, 4><<<grid, threads, lds, stream>>>(
           (float*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
           (float*)k_cache, (float*)v_cache, nheads, kvheads, head_dim, n_tokens);
+    else if (by_eights)
+      rope_kv_tile_kernel<bf16, 8><<<grid, threads, lds, stream>>>(
+          (bf16*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
+          (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim, n_tokens);
     else
-      rope_kv_tile_kernel<bf16><<<grid, threads, lds, stream>>>(
+      rope_kv_tile_kernel<bf16, 4><<<grid, threads, lds, stream>>>(
           (bf16*)qkv, row_stride, positions, seq_of_token, block_table, table_stride, c, sin_t, rot_dim, max_pos,
           (bf16*)k_cache, (bf16*)v_cache, nheads, kvheads, head_dim, n_tokens);
   } else if (dtype == FMS_F32)

@@ -143,9 +143,11 @@ def fill_cache(table, ks, vs, n_pages, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,K,D,rot", [(4, 2, 16, 16), (3, 1, 24, 24), (2, 2, 32, 16), (2, 1, 6, 6), (8, 2, 128, 128), (3, 3, 256, 64)])
-def test_rope_kv_write(ops, dtype, H, K, D, rot):
+@pytest.mark.parametrize("starts,lens", [([0, 70, 5], [9, 3, 130]), ([0, 64, 8, 3], [200, 72, 56, 13])])
+def test_rope_kv_write(ops, dtype, H, K, D, rot, starts, lens):
+    """The second layout has runs of tokens that start at multiples of 8 places of their pages and cross page
+    borders (whole 16-byte pieces of the transposed value pages), the first has none to speak of."""
     torch.manual_seed(4)
-    starts, lens = [0, 70, 5], [9, 3, 130]
     total = [s + n for s, n in zip(starts, lens)]
     table, n_pages = make_pages(total, K, D, dtype, seed=1)
     T = sum(lens)
