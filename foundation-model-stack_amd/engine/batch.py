@@ -36,6 +36,9 @@ class StepBatch:
     # decode steps: the token rows from the longest context to the shortest (int32 [T]).  A kernel whose blocks
     # take a sequence each hands out the long ones first, so that none of them is left to run alone at the end.
     rows_by_length: Optional[torch.Tensor] = None
+    # Rows of the logits that the caller asked for: the first n_wanted of the n_logit_rows that are computed (a
+    # decode step padded to a row bucket computes a row for every padding token as well, as a captured step does).
+    n_wanted: int = 0
 
 
 def build_batch(
@@ -46,9 +49,13 @@ def build_batch(
     want: Sequence[Sequence[int]],
     device,
     qblock_sizes: Sequence[int] = (),
+    pad_rows_to: int = 0,
 ) -> StepBatch:
     """Index arrays of a step.  `starts[b]` is what cache.extend(slot, len(tokens[b])) returned.
-    qblock_sizes: the block sizes in which mixers want the step's tokens cut (blocks never span sequences)."""
+    qblock_sizes: the block sizes in which mixers want the step's tokens cut (blocks never span sequences).
+    pad_rows_to: a decode step (one token a sequence) is filled up to this many token rows with padding rows
+    (sequence -1, which every kernel skips), so that it has the shape of the captured step of that many rows:
+    the same kernels then run with the same launch, and give the same bits."""
     B = len(slots)
     q_lens = [len(t) for t in tokens]
     T = sum(q_lens)
@@ -79,6 +86,17 @@ def build_batch(
     # one host buffer, one copy
     is_decode = all(n == 1 for n in q_lens)
     by_length = np.argsort(-positions, kind="stable") if is_decode else []
+    n_wanted = len(rows)
+    pad = pad_rows_to - T if is_decode and B and pad_rows_to > T else 0
+    if pad:
+        filler = np.zeros(pad, dtype=np.int64)
+        flat_ids = np.concatenate([flat_ids, filler])
+        positions = np.concatenate([positions, filler])
+        seq_of_token = np.concatenate([seq_of_token, filler - 1])
+        by_length = np.concatenate([by_length, np.arange(T, T + pad)])
+        if rows == list(range(T)):  # every sequence's token is wanted: the padding rows' too, as in a captured step
+            rows = rows + list(range(T, T + pad))
+        T += pad
     parts = [flat_ids, positions, seq_of_token, list(slots), seq_starts, rows, by_length]
     for size in sizes:
         parts += [qb_start[size], qb_len[size]]
@@ -123,4 +141,5 @@ def build_batch(
         logit_rows=span(5),
         n_logit_rows=len(rows),
         rows_by_length=span(6) if is_decode else None,
+        n_wanted=n_wanted,
     )

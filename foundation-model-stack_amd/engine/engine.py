@@ -41,7 +41,12 @@ class Engine:
         self.vocab = model.spec.vocab
         if use_graphs is None:
             use_graphs = not os.environ.get("FMS_AMD_NO_GRAPHS")
-        self.use_graphs = bool(use_graphs) and all(getattr(p, "graph_safe", True) for p in model.walk())
+        capturable = all(getattr(p, "graph_safe", True) for p in model.walk())
+        self.use_graphs = bool(use_graphs) and capturable
+        # Eager decode steps take the shape of the captured step of their row bucket (padding rows of sequence -1),
+        # if every part knows such rows: eager steps and replays then run the same kernels with the same launches
+        # and give the same bits.
+        self.pads_decode_rows = capturable
         self._graphs = {}
         self.graph_captures = []  # (rows, context bound) of every capture, in order
         self.last_graph: Optional[DecodeGraph] = None  # the graph of the last replayed step (its .logits are that step's)
@@ -71,7 +76,8 @@ class Engine:
         batch = self.prepare(slots, tokens, want)
         if batch.n_tokens == 0:
             return torch.empty(0, self.vocab, dtype=torch.float32, device=self.device)
-        return self.model.forward(batch, self.cache)
+        logits = self.model.forward(batch, self.cache)
+        return logits if batch.n_wanted == batch.n_logit_rows else logits[: batch.n_wanted]
 
     def decode_and_choose(
         self,
@@ -148,7 +154,8 @@ class Engine:
                 size = block.mixer.prefill_qblock(n_tokens, self.model.dtype)
                 if size:
                     sizes.add(size)
-        batch = build_batch(self.cache, slots, tokens, starts, want, self.device, sizes)
+        pad_to = row_bucket(len(slots)) if self.pads_decode_rows and all(len(t) == 1 for t in tokens) else 0
+        batch = build_batch(self.cache, slots, tokens, starts, want, self.device, sizes, pad_rows_to=pad_to)
         if batch.is_decode:
             # the bound a graph for this step would be captured for: eager steps and replays then launch the
             # same kernels in the same shape, and give the same bits

@@ -518,6 +518,37 @@ def test_graph_for_a_longer_context_replaces_the_shorter_one(lib, folders, dtype
         assert (4, 2048) in captured and (4, 4096) in captured and captured.index((4, 2048)) < captured.index((4, 4096))
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "E"])
+def test_replayed_and_eager_steps_choose_the_same_tokens(lib, folders, name, dtype):
+    """An eager decode step has the shape of the captured step of its row bucket (padding rows, the same context
+    bound), so both run the same kernels with the same launches: generation through graphs and through eager steps
+    gives the same tokens, bit for bit, greedy and sampled, while sequences end at different times and the batch
+    shrinks from one row bucket to the next.  Any index that a graph kept past its time would show here."""
+    from fms_amd.engine import Engine
+    from fms_amd.generation import generate_requests
+    from fms_amd.sampling import SamplingParams
+
+    model = get(lib, folders, name, dtype)
+    lens = varied_lengths(37, 120)
+    prompts = [tokens_for(name, n, 900 + i) for i, n in enumerate(lens)]
+    room = sum(-(-(n + 90) // 64) * 64 for n in lens)
+    stops = list(range(3, CONFIGS[name]["src_vocab_size"], 23))  # about one token in 23 ends its sequence
+    got = {}
+    for graphs in (True, False):
+        engine = Engine(model, max_tokens=room, max_slots=len(lens), use_graphs=graphs)
+        assert engine.use_graphs == graphs
+        for sampling in (SamplingParams(do_sample=False), SamplingParams(do_sample=True, temperature=0.9, top_k=20)):
+            got[(graphs, sampling.do_sample)] = generate_requests(engine, prompts, max_new_tokens=90, sampling=sampling, seed=5,
+                                                                  stop_token_ids=stops)
+        engine.cache.check()
+        if graphs:
+            assert len(set(engine.graph_captures)) >= 3  # the batch went through several row buckets
+    for sampled in (False, True):
+        assert got[(True, sampled)] == got[(False, sampled)]
+        assert len(set(len(g) for g in got[(True, sampled)])) > 3  # they ended at different times
+
+
 # --------------------------------------------------------------------------
 def varied_lengths(n, longest):
     """n prompt lengths between 1 and `longest`, among them the neighbours of the page borders."""

@@ -502,10 +502,23 @@ def test_a_decode_batch_lists_its_rows_longest_context_first():
     starts = [cache.extend(slot, 1) for slot in slots]
     batch = build_batch(cache, slots, [[1], [2], [3], [4]], starts, [[0]] * 4, "cpu")
     assert batch.is_decode and batch.rows_by_length.tolist() == [1, 3, 2, 0]
+    assert batch.n_tokens == 4 and batch.n_wanted == 4 == batch.n_logit_rows
+    # filled up to the rows of a captured step: padding rows of sequence -1 at the end, which are computed and not wanted
+    more = [cache.extend(slot, 1) for slot in slots]
+    padded = build_batch(cache, slots, [[1], [2], [3], [4]], more, [[0]] * 4, "cpu", pad_rows_to=8)
+    assert padded.n_tokens == 8 and padded.n_seqs == 4 and padded.n_wanted == 4 and padded.n_logit_rows == 8
+    assert padded.seq_of_token.tolist() == [0, 1, 2, 3, -1, -1, -1, -1] and padded.token_ids.tolist() == [1, 2, 3, 4, 0, 0, 0, 0]
+    assert padded.positions.tolist()[:4] == more and padded.rows_by_length.tolist() == [1, 3, 2, 0, 4, 5, 6, 7]
+    assert padded.logit_rows.tolist() == list(range(8)) and padded.max_context == max(more) + 1
+    # where only some rows are wanted, nothing is computed for padding rows
+    few = build_batch(cache, slots, [[1], [2], [3], [4]], [cache.extend(slot, 1) for slot in slots], [[0], [], [0], []], "cpu", pad_rows_to=8)
+    assert few.n_tokens == 8 and few.logit_rows.tolist() == [0, 2] and few.n_wanted == 2 == few.n_logit_rows
     # a step that brings a prompt has no such order
     other = cache.alloc_slot()
     batch = build_batch(cache, [other], [[1, 2, 3]], [cache.extend(other, 3)], [[2]], "cpu")
     assert not batch.is_decode and batch.rows_by_length is None
+    batch = build_batch(cache, [other], [[1, 2]], [cache.extend(other, 2)], [[1]], "cpu", pad_rows_to=8)
+    assert batch.n_tokens == 2  # only decode steps are filled up
 
 
 # --------------------------------------------------------------------------

@@ -192,6 +192,31 @@ def test_decode_batches_through_graphs(shape, n_seqs):
         assert error <= MARGIN * largest, f"sequence {i} ({s['n']} prompt tokens): bfloat16 is {error:.4g} from float32"
 
 
+def test_replayed_and_eager_steps_choose_the_same_tokens(shape):
+    """At these sizes too (the products for 17 to 128 rows cut K by the number of rows, the decode attention splits
+    by it): an eager decode step is filled up to the rows of the captured step, so generation through graphs and
+    through eager steps gives the same tokens bit for bit while the batch shrinks through the row buckets."""
+    from fms_amd.engine import Engine
+    from fms_amd.generation import generate_requests
+    from fms_amd.sampling import SamplingParams
+
+    model = shape.model("bfloat16")
+    lens = prompt_lengths(45)
+    prompts = [shape.tokens(n, 3000 + i) for i, n in enumerate(lens)]
+    room = sum(-(-(n + 60) // 64) * 64 for n in lens)
+    stops = list(range(5, shape.cfg.vocab, 19))
+    got = {}
+    for graphs in (True, False):
+        engine = Engine(model, max_tokens=room, max_slots=len(lens), use_graphs=graphs)
+        for sampling in (SamplingParams(do_sample=False), SamplingParams(do_sample=True, temperature=0.8, top_k=10)):
+            got[(graphs, sampling.do_sample)] = generate_requests(engine, prompts, max_new_tokens=60, sampling=sampling, seed=9,
+                                                                  stop_token_ids=stops)
+        engine.cache.check()
+        if graphs:
+            assert len(set(engine.graph_captures)) >= 4
+    assert got[(True, False)] == got[(False, False)] and got[(True, True)] == got[(False, True)]
+
+
 # ---- depth ------------------------------------------------------------------------------------------------------
 DEEP = dict(src_vocab_size=4096, emb_dim=1024, nheads=8, kvheads=2, nlayers=32, hidden_dim=3584, multiple_of=1,
             norm_eps=1e-5, rope_theta=500000.0, max_expected_seq_len=2048)
