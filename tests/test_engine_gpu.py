@@ -519,6 +519,37 @@ def test_graph_for_a_longer_context_replaces_the_shorter_one(lib, folders, dtype
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "E"])
+def test_logits_do_not_depend_on_the_place_in_the_cache(lib, folders, name, dtype):
+    """The same sequence in a fresh cache (slot 0, pages 0, 1, 2, ...) and in one that other sequences have used
+    and partly left (another slot, pages out of order that still hold the others' keys and values): the same
+    kernels add the same numbers in the same order, so the logits are the same bits."""
+    from fms_amd.engine import Engine
+
+    model = get(lib, folders, name, dtype)
+    ids = tokens_for(name, 300, 77)
+
+    def run(others):
+        engine = Engine(model, max_tokens=64 * 24, max_slots=8, use_graphs=False)
+        held = []
+        for i, n in enumerate(others):
+            held.append(engine.new_sequence())
+            engine.step([held[-1]], [tokens_for(name, n, 200 + i)], "last")
+        for slot in held[::2]:
+            engine.end_sequence(slot)
+        slot = engine.new_sequence()
+        out = [engine.step([slot], [ids[:200]], "all")]
+        for tok in ids[200:]:
+            out.append(engine.step([slot], [[tok]], "last"))
+        return torch.cat(out), slot, list(engine.cache.groups[0].pages[slot])
+
+    fresh, slot_a, pages_a = run([])
+    used, slot_b, pages_b = run([100, 70, 129, 5, 64])
+    assert slot_a != slot_b and pages_a != pages_b and pages_b != sorted(pages_b)
+    assert torch.equal(fresh, used)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", ["A", "E"])
 def test_replayed_and_eager_steps_choose_the_same_tokens(lib, folders, name, dtype):
     """An eager decode step has the shape of the captured step of its row bucket (padding rows, the same context
