@@ -307,6 +307,91 @@ def test_a_layer_named_twice_and_a_layer_reading_another_cache(lib, tmp_path):
     torch.testing.assert_close(torch.cat(got).cpu(), plain(ids), atol=2e-4, rtol=1e-3)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_a_layer_with_a_window_among_layers_without(lib, dtype):
+    """Layers are configured one by one: Llama's parts with a window of 70 keys in the middle layer only.  That layer
+    has a cache group of its own, which gives pages back while the sequences grow (the others keep theirs).  Two
+    sequences of unequal lengths, a prompt step and 150 decode steps, as eager steps and through captured graphs,
+    against the plain parts; the bfloat16 run against the float32 one."""
+    import copy
+
+    import fms_amd
+    from fms_amd.architectures.llama import llama_spec
+    from fms_amd.engine import Engine
+    from fms_amd.engine.model import DecoderModel
+    from fms_amd.sampling import SamplingParams
+    from fms_amd.weights import init_random
+
+    WINDOW = 70
+    config = fms_amd.LLaMAConfig(src_vocab_size=120, emb_dim=64, nheads=4, kvheads=2, nlayers=3, hidden_dim=96, multiple_of=1,
+                                 max_expected_seq_len=512)
+    spec = llama_spec(config)
+    spec.layers = [copy.deepcopy(layer) for layer in spec.layers]
+    spec.layers[1].mixer.args["window"] = WINDOW
+    model = DecoderModel(spec, dtype, config=config)
+    init_random(model, 9, torch.device(DEV), std=0.1, norm_std=0.1)
+    model.finalize_all(DEV)
+    kv, _ = model.cache_needs()
+    assert sorted(need.window for _, need in kv) == [0, 0, WINDOW]
+    w = {name: owner.w[local].float().cpu() for name, _, owner, local in model.named_specs()}
+
+    def plain(ids):
+        S = len(ids)
+        pos = torch.arange(S)
+        freqs = P.rope_frequencies(16, 1e4)
+        x = w["base_model.embedding.weight"][torch.tensor(ids)]
+        for layer in range(3):
+            p = f"base_model.layers.{layer}."
+            h = P.rms_norm(x, w[p + "ln.weight"], 1e-5)
+            qkv = h @ w[p + "attn.in_proj.qkv_fused.weight"].t()
+            q, k, v = torch.split(qkv, [64, 32, 32], dim=-1)
+            q = P.rope_rotate(q.reshape(S, 4, 16), pos, freqs)
+            k = P.rope_rotate(k.reshape(S, 2, 16), pos, freqs)
+            a = P.causal_attention(q, k, v.reshape(S, 2, 16), window=WINDOW if layer == 1 else 0)
+            x = x + a.reshape(S, 64) @ w[p + "attn.dense.weight"].t()
+            h = P.rms_norm(x, w[p + "ff_ln.weight"], 1e-5)
+            x = x + P.gated_feed_forward(h, w[p + "ff_sub_layer.wg1_fused.weight"], w[p + "ff_sub_layer.w2.weight"])
+        return P.rms_norm(x, w["base_model.dec_norm.weight"], 1e-5) @ w["head.weight"].t()
+
+    g = torch.Generator().manual_seed(4)
+    seqs = [torch.randint(0, 120, (n,), generator=g).tolist() for n in (290, 215)]
+    prompt = (140, 65)
+    want = [plain(ids) for ids in seqs]
+    greedy = SamplingParams(do_sample=False)
+    for graphs in (False, True):
+        engine = Engine(model, max_tokens=64 * 12, max_slots=2, use_graphs=graphs)
+        assert engine.use_graphs == graphs
+        slots = [engine.new_sequence() for _ in seqs]
+        logits = engine.step(slots, [ids[:n] for ids, n in zip(seqs, prompt)], "all")
+        got = [[logits[: prompt[0]]], [logits[prompt[0] :]]]
+        windowed = [i for i, group in enumerate(engine.cache.groups) if group.need.window][0]
+        held_at_start = [len([p for p in engine.cache.groups[windowed].pages[s] if p >= 0]) for s in slots]
+        for step in range(150):
+            fed = [ids[n + step] for ids, n in zip(seqs, prompt)]
+            if graphs:
+                engine.decode_and_choose(slots, fed, greedy)
+                rows = engine.last_graph.logits[:2].float()
+            else:
+                rows = engine.step(slots, [[t] for t in fed], "last")
+            got[0].append(rows[0:1].clone())
+            got[1].append(rows[1:2].clone())
+        # the windowed group let pages go while the sequences grew by 150 tokens; the others hold every page
+        full = [i for i, group in enumerate(engine.cache.groups) if not group.need.window][0]
+        for b, s in enumerate(slots):
+            live = [p for p in engine.cache.groups[windowed].pages[s] if p >= 0]
+            assert len(live) <= 3 and len(live) <= held_at_start[b] + 1
+            assert len([p for p in engine.cache.groups[full].pages[s] if p >= 0]) == -(-(prompt[b] + 150) // 64)
+        engine.cache.check()
+        for s in slots:
+            engine.end_sequence(s)
+        for rows, ref in zip(got, want):
+            out = torch.cat(rows).cpu()
+            if dtype == torch.float32:
+                torch.testing.assert_close(out, ref, atol=2e-4, rtol=1e-3)
+            else:
+                assert float((out - ref).abs().max()) <= 0.06 * float(ref.abs().max())
+
+
 def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(lib):
     """Two more kinds of part that the library does not have, defined here and registered by name:
     a feed-forward that routes every token to one of three small experts (router logits and the chosen
