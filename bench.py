@@ -5,7 +5,9 @@
 Random weights, synthetic token ids.  A "step" is one decode step of the whole batch through
 the library's own generation path (step function, cache, kernels, sampler).  One JSON line is
 printed: decode tokens/s at batch 8 (`value`), the prefill of 2,048 tokens, the decode step's
-memory roofline, and decode at batch 1 and 64.
+memory roofline (against the published peak and against what a pure read reaches on this GPU now),
+the share of the step's time by kernel class, and further points: decode at batch 1 and 64, at
+batch 8 with every context near 8000 tokens, and the Llama-2-7B shape at batch 8 (256 steps).
 """
 
 import argparse
@@ -35,7 +37,9 @@ def main() -> int:
     ap.add_argument("--prefill-tokens", type=int, default=2048)
     ap.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
     ap.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches")
-    ap.add_argument("--skip-points", action="store_true", help="leave out decode at batch 1 and 64")
+    ap.add_argument("--skip-points", action="store_true", help="leave out the further points (batch 1 and 64, long contexts, the 7B shape)")
+    ap.add_argument("--with-70b", action="store_true",
+                    help="add the Llama-3-70B shape at batch 16, prompts of 256..4096, 128 steps (141 GB of weights: minutes)")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="run one phase only (for profiling); the record then lacks the other")
@@ -59,7 +63,11 @@ def main() -> int:
     import fms_amd
     from fms_amd.architectures import variant_config
     from fms_amd.engine import Engine
+    from fms_amd.kernels import ops
     from fms_amd.sampling import SamplingParams, choose
+
+    # what this GPU delivers now: a kernel that only reads, a kernel that only issues matrix instructions
+    read_bps, mfma_flops = ops.measured_peaks()
 
     full = variant_config("llama", args.variant)
     overrides = {"max_expected_seq_len": args.context}
@@ -69,20 +77,29 @@ def main() -> int:
     cfg = model.config
     E, H, K, D, F, V, L = (cfg.emb_dim, cfg.nheads, cfg.kv_heads, cfg.head_dim, cfg.ffn_hidden_dim, cfg.src_vocab_size,
                            cfg.nlayers)
-    layer_weights = (H + 2 * K) * D * E + E * H * D + 2 * F * E + E * F + 2 * E  # elements per layer, norms included
-    step_weight_bytes = 2 * (L * layer_weights + E + V * E)  # everything but the embedding table, read once
-    kv_bytes_per_token = 2 * L * K * D * 2
+
+    def step_bytes_of(c):
+        """(bytes of weights a decode step reads: everything but the embedding table, once; cache bytes per token)"""
+        e, h, k, d, f = c.emb_dim, c.nheads, c.kv_heads, c.head_dim, c.ffn_hidden_dim
+        layer = (h + 2 * k) * d * e + e * h * d + 2 * f * e + e * f + 2 * e  # elements per layer, norms included
+        return 2 * (c.nlayers * layer + e + c.src_vocab_size * e), 2 * c.nlayers * k * d * 2
+
+    step_weight_bytes, kv_bytes_per_token = step_bytes_of(cfg)
     greedy = SamplingParams(do_sample=False)
     rng = random.Random(args.seed)
 
-    def decode(batch: int, steps: int, warmup: int):
-        """(tokens/s, ms per step, bytes a step has to read) for `batch` sequences with prompts of 128..2048 tokens."""
-        lens = [rng.randint(args.prompt_min, args.prompt_max) for _ in range(batch)]
-        room = sum(-(-(n + steps + warmup + 1) // 64) * 64 for n in lens)
+    def decode(batch: int, steps: int, warmup: int, model=model, prompt_min=args.prompt_min, prompt_max=args.prompt_max,
+               shares=None):
+        """(tokens/s, ms per step, bytes a step has to read) for `batch` sequences with prompts of prompt_min..prompt_max
+        tokens.  shares: a dict that takes the share of an eager step's time by kernel class."""
+        weight_bytes, kv_bytes = step_bytes_of(model.config)
+        V = model.config.src_vocab_size
+        lens = [rng.randint(prompt_min, prompt_max) for _ in range(batch)]
+        room = sum(-(-(n + steps + warmup + 8) // 64) * 64 for n in lens)
         engine = Engine(model, max_tokens=room, max_slots=batch)
         slots = [engine.new_sequence() for _ in range(batch)]
         tokens = None
-        per_group = max(1, 16384 // args.prompt_max)  # prompts in groups, so that activations stay small
+        per_group = max(1, 16384 // prompt_max)  # prompts in groups, so that activations stay small
         for i in range(0, batch, per_group):
             group = list(range(i, min(i + per_group, batch)))
             prompts = [[rng.randrange(V) for _ in range(lens[b])] for b in group]
@@ -98,11 +115,52 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         mean_ctx = sum(lens) + batch * (1 + warmup + steps / 2)
+        if shares is not None:
+            shares.update(kernel_shares(engine, slots, tokens))
         for s in slots:
             engine.end_sequence(s)
         del engine
         torch.cuda.empty_cache()
-        return batch * steps / dt, 1000 * dt / steps, step_weight_bytes + kv_bytes_per_token * mean_ctx
+        return batch * steps / dt, 1000 * dt / steps, weight_bytes + kv_bytes * mean_ctx
+
+    def kernel_shares(engine, slots, tokens):
+        """The share of a decode step's GPU time by kernel class: three eager steps (the same kernels in the same
+        shape as the replayed graph) with an event before and after every call into the kernel library."""
+        classes = {"qkv_rope_write": "qkv_rope_cache", "attention": "attention", "gated_linear": "gate_up_act",
+                   "sample": "sampling", "embed": "other", "add_norm": "other", "advance_positions_": "other"}
+        spans, originals = [], {}
+
+        def timed(name, fn):
+            def call(*a, **kw):
+                kind = classes.get(name)
+                if name == "linear_into_stream":
+                    kind = "o_proj_residual" if a[0].shape[1] == a[1].shape[0] else "down_residual"
+                if name == "linear":
+                    kind = "head" if a[1].shape[0] == engine.vocab else "other"
+                first, last = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                first.record()
+                out = fn(*a, **kw)
+                last.record()
+                spans.append((kind, first, last))
+                return out
+            return call
+
+        for name in list(classes) + ["linear_into_stream", "linear"]:
+            originals[name] = getattr(ops, name)
+            setattr(ops, name, timed(name, originals[name]))
+        try:
+            for _ in range(3):
+                logits = engine.step(slots, [[t] for t in tokens], "last")
+                tokens = choose(logits, greedy).tolist()
+            torch.cuda.synchronize()
+        finally:
+            for name, fn in originals.items():
+                setattr(ops, name, fn)
+        total = {}
+        for kind, first, last in spans:
+            total[kind] = total.get(kind, 0.0) + first.elapsed_time(last)
+        whole = sum(total.values()) or 1.0
+        return {kind: round(ms / whole, 4) for kind, ms in sorted(total.items())}
 
     def prefill(n_tokens: int):
         engine = Engine(model, max_tokens=n_tokens + 64, max_slots=1)
@@ -122,25 +180,44 @@ def main() -> int:
         flops = 2.0 * n_tokens * L * ((H + 2 * K) * D * E + E * H * D + 2 * F * E + E * F)
         flops += L * 4.0 * H * D * n_tokens * (n_tokens + 1) / 2  # causal scores and mixing
         flops += 2.0 * E * V  # the head for one row
-        return n_tokens / t, 1000 * t, flops / t / PEAK_FLOPS["bf16"]
+        return n_tokens / t, 1000 * t, flops / t / PEAK_FLOPS["bf16"], flops / t / mfma_flops
 
-    pre_tps = pre_ms = pre_frac = 0.0
+    pre_tps = pre_ms = pre_frac = pre_frac_measured = 0.0
     tps = ms = step_bytes = 0.0
+    shares = {}
     if args.only != "decode":
-        pre_tps, pre_ms, pre_frac = prefill(args.prefill_tokens)
+        pre_tps, pre_ms, pre_frac, pre_frac_measured = prefill(args.prefill_tokens)
     if args.only != "prefill":
-        tps, ms, step_bytes = decode(args.batch, args.steps, args.warmup)
+        tps, ms, step_bytes = decode(args.batch, args.steps, args.warmup, shares=shares)
     achieved = step_bytes / (ms / 1000) / 1e9 if ms else 0.0
     points = {}
+
+    def point(name, p_tps, p_ms, p_bytes):
+        gbs = p_bytes / (p_ms / 1000) / 1e9
+        points[name] = round(p_tps, 1)
+        points[f"{name}_ms"] = round(p_ms, 3)
+        points[f"{name}_gb"] = round(p_bytes / 1e9, 3)
+        points[f"{name}_gbs"] = round(gbs, 1)
+        points[f"{name}_frac"] = round(gbs / HBM_GBS, 4)
+
     if not args.skip_points and args.only is None:
         for b, steps, warmup in ((1, min(args.steps, 32), 4), (64, min(args.steps, 16), 2)):
-            p_tps, p_ms, p_bytes = decode(b, steps, warmup)
-            gbs = p_bytes / (p_ms / 1000) / 1e9
-            points[f"decode_b{b}"] = round(p_tps, 1)
-            points[f"decode_b{b}_ms"] = round(p_ms, 3)
-            points[f"decode_b{b}_gb"] = round(p_bytes / 1e9, 3)
-            points[f"decode_b{b}_gbs"] = round(gbs, 1)
-            points[f"decode_b{b}_frac"] = round(gbs / HBM_GBS, 4)
+            point(f"decode_b{b}", *decode(b, steps, warmup))
+        # every context near the benchmark's context length
+        near = min(8000, args.context - 64)
+        point(f"decode_b8_ctx{near}", *decode(8, min(args.steps, 16), 2, prompt_min=near - 100, prompt_max=near))
+        # the Llama-2-7B shape: batch 8, prompts of 64..1024 tokens, 256 decode steps, context 4096
+        other = fms_amd.get_model("llama", "2-7b", data_type="bf16", device_type="cuda", random_seed=args.seed,
+                                  max_expected_seq_len=4096)
+        point("llama2_7b_b8", *decode(8, 256, 8, model=other, prompt_min=64, prompt_max=1024))
+        del other
+        torch.cuda.empty_cache()
+        if args.with_70b:
+            big = fms_amd.get_model("llama", "3-70b", data_type="bf16", device_type="cuda", random_seed=args.seed,
+                                    max_expected_seq_len=8192)
+            point("llama3_70b_b16", *decode(16, 128, 4, model=big, prompt_min=256, prompt_max=4096))
+            del big
+            torch.cuda.empty_cache()
 
     record = {
         "metric": f"decode tok/s at batch {args.batch} (llama {args.variant} shape, {args.context} context); prefill tok/s at {args.prefill_tokens} tokens",
@@ -175,9 +252,12 @@ def main() -> int:
             "prefill_tokens": args.prefill_tokens,
             "cache_page_tokens": 64,
         },
-        "prefill": {"value": round(pre_tps, 1), "tokens": args.prefill_tokens, "ms": round(pre_ms, 3), "frac": round(pre_frac, 4)},
+        "prefill": {"value": round(pre_tps, 1), "tokens": args.prefill_tokens, "ms": round(pre_ms, 3), "frac": round(pre_frac, 4),
+                    "frac_measured": round(pre_frac_measured, 4), "peak_measured_tflops": round(mfma_flops / 1e12, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_GBS, 4)},
+                     "frac": round(achieved / HBM_GBS, 4), "peak_measured": round(read_bps / 1e9, 1),
+                     "frac_measured": round(achieved / (read_bps / 1e9), 4)},
+        "shares": shares,
         "points": points,
     }
     print(json.dumps(record))

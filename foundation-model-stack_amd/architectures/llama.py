@@ -139,12 +139,27 @@ register_adapter(NAME, "hf", ["hf_to_fms_names", "hf_to_fms_rope", "weight_fusio
 register_adapter(NAME, "fms_unfused", ["weight_fusion"])
 
 
+def _pre006_attention_names(sd, **kw):
+    """Checkpoints written before the reference's 0.0.6 name the projections attn.query/key/value, without
+    "in_proj" (fms/utils/serialization.py:164-170, 182-227 with attn_prefix="attn")."""
+    pattern = re.compile(r"\.attn\.(query|key|value)\.(weight|bias)$")
+    return {pattern.sub(r".attn.in_proj.\1.\2", name): t for name, t in sd.items()}
+
+
+register_adapter_step(NAME, "pre0.0.6_attn_unfused_to_fused", lambda sd, **kw: fuse_attention_step(_pre006_attention_names(sd)))
+register_adapter_step(NAME, "swiglu_unfused_to_fused", fuse_glu_step)
+# fms/models/llama.py:761-765
+register_adapter(NAME, "fms.pre0.0.6", ["pre0.0.6_attn_unfused_to_fused", "swiglu_unfused_to_fused", "weight_fusion"])
+
+
 def detect_source(names: List[str]) -> str:
     """Which source a checkpoint's tensor names come from."""
     if any(n.startswith("model.layers.") or n.startswith("model.embed_tokens") for n in names):
         return "hf"
     if any(n.startswith("tok_embeddings") or ".attention.wq" in n for n in names):
         return "meta"
+    if any(re.search(r"\.attn\.(query|key|value)\.", n) for n in names):
+        return "fms.pre0.0.6"
     if any(".in_proj.query." in n or ".ff_sub_layer.wg." in n for n in names):
         return "fms_unfused"
     return "fms"

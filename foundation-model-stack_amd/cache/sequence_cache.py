@@ -52,6 +52,9 @@ class KVGroup:
         self.values: Optional[torch.Tensor] = None
         # slot -> logical page list; -1 marks a page given back because the window has passed it
         self.pages: Dict[int, List[int]] = {}
+        # slot -> index of the slot's first page that has not been given back (everything before it is -1): a
+        # window's releases are looked for from there, not from the sequence's start, at every step
+        self.first_held: Dict[int, int] = {}
 
     def allocate_storage(self, dtype: torch.dtype, device) -> None:
         n, K, D = self.pool.n_pages, self.need.kv_heads, self.need.head_dim
@@ -126,6 +129,7 @@ class SequenceCache:
         self._stamp[slot] = self._clock
         for group in self.groups:
             group.pages[slot] = []
+            group.first_held[slot] = 0
         for tensors in self.state.values():
             for t in tensors.values():
                 t[slot].zero_()
@@ -138,6 +142,7 @@ class SequenceCache:
             for page in group.pages.pop(slot):
                 if page >= 0:
                     group.pool.free(page)
+            group.first_held.pop(slot, None)
         del self._live[slot]
         del self._stamp[slot]
         self._free_slots.append(slot)
@@ -178,7 +183,7 @@ class SequenceCache:
             release = []
             if group.need.window > 0:
                 first_visible = max(0, start - group.need.window + 1)
-                release = [i for i in range(min(first_visible // PAGE_TOKENS, len(pages))) if pages[i] >= 0]
+                release = list(range(group.first_held[slot], min(first_visible // PAGE_TOKENS, len(pages))))
             plans.append((group, release, max(0, pages_for(new_len) - len(pages))))
         return plans
 
@@ -204,6 +209,8 @@ class SequenceCache:
                 for i in release:
                     group.pool.free(pages[i])
                     pages[i] = -1
+                if release:
+                    group.first_held[slot] = release[-1] + 1
         for slot, n, plan in zip(slots, new_tokens, plans):
             for group, _, want in plan:
                 pages = group.pages[slot]
@@ -223,7 +230,14 @@ class SequenceCache:
     def stamp(self, slot: int) -> int:
         """A number that changes whenever the slot is handed out or its sequence grows, and never comes back:
         who remembers it can tell whether the sequence is still as they left it."""
+        if slot not in self._stamp:
+            raise ValueError(f"slot {slot} is not live")
         return self._stamp[slot]
+
+    def pages_held(self, slot: int) -> int:
+        """How many pages the slot holds over all groups: it changes when the sequence gets a page and when a
+        window gives one back, so whoever keeps a copy of the block tables knows when to read them again."""
+        return sum(len(group.pages[slot]) - group.first_held[slot] for group in self.groups)
 
     def block_table(self, group_index: int, slots: Sequence[int], n_columns: Optional[int] = None) -> torch.Tensor:
         """int32 [len(slots), n_columns] page numbers on the host (unused entries and released pages: -1)."""
@@ -267,3 +281,7 @@ class SequenceCache:
                 raise AssertionError("pages held by sequences and by the pool differ")
             if set(group.pages) != set(self._live):
                 raise AssertionError("page lists and live slots differ")
+            for slot, pages in group.pages.items():
+                first = group.first_held[slot]
+                if any(p >= 0 for p in pages[:first]) or any(p < 0 for p in pages[first:]):
+                    raise AssertionError("released pages are not exactly the pages before the first held one")

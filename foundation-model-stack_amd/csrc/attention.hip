@@ -21,12 +21,16 @@
 // ==========================================================================
 #define GEN_THREADS 256
 
-template <typename T>
+// TERMS: the scores carry further terms (fms/modules/positions.py:9-36, the reference's adjusted_mask): a soft cap
+// cap * tanh(score / cap), and a bias slope[head] * (key position - query position), which is zero or negative.
+// Without TERMS neither is compiled in.
+template <typename T, bool TERMS>
 __global__ void __launch_bounds__(GEN_THREADS)
     attn_generic_kernel(const T* __restrict__ q, long q_stride, T* __restrict__ out, long out_stride,
                         const int* __restrict__ positions, const int* __restrict__ seq_of_token,
                         const int* __restrict__ block_table, int table_stride, const T* __restrict__ k_cache,
-                        const T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale, int window) {
+                        const T* __restrict__ v_cache, int nheads, int kvheads, int head_dim, float scale, int window,
+                        const float* __restrict__ slopes, float soft_cap) {
   __shared__ float qs[256];
   __shared__ float ps[GEN_THREADS];
   __shared__ float scratch[17];
@@ -58,6 +62,10 @@ __global__ void __launch_bounds__(GEN_THREADS)
       float dot = 0.f;
       for (int d = 0; d < head_dim; ++d) dot = fmaf(qs[d], to_f32(krow[d]), dot);
       s = dot * scale;
+      if (TERMS) {
+        if (soft_cap > 0.f) s = soft_cap * tanhf(s / soft_cap);
+        if (slopes != nullptr) s = fmaf(slopes[h], (float)(j - pos), s);
+      }
     }
     const float m_new = fmaxf(m_run, block_max(s, scratch));
     const float p = j <= pos ? expf(s - m_new) : 0.f;
@@ -993,21 +1001,31 @@ extern "C" int fmsamd_attn_generic(const void* q, long q_stride, void* out, long
                                    const int* positions, const int* seq_of_token, const int* block_table,
                                    int table_stride, const void* k_cache, const void* v_cache, int n_tokens,
                                    int nheads, int kvheads, int head_dim, float scale, int window,
-                                   hipStream_t stream) {
+                                   const float* slopes, float soft_cap, hipStream_t stream) {
   if (n_tokens == 0) return 0;
   if (check_common("attn_generic", n_tokens, nheads, kvheads, head_dim, q_stride, out_stride)) return -1;
   FMS_REQUIRE(n_tokens <= 65535, "attn_generic: %d tokens exceed one launch (65535)", n_tokens);
+  FMS_REQUIRE(soft_cap >= 0.f, "attn_generic: soft cap %g is negative", (double)soft_cap);
   dim3 grid(nheads, n_tokens);
-  if (dtype == FMS_F32)
-    attn_generic_kernel<float><<<grid, GEN_THREADS, 0, stream>>>(
-        (const float*)q, q_stride, (float*)out, out_stride, positions, seq_of_token, block_table, table_stride,
-        (const float*)k_cache, (const float*)v_cache, nheads, kvheads, head_dim, scale, window);
-  else if (dtype == FMS_BF16)
-    attn_generic_kernel<bf16><<<grid, GEN_THREADS, 0, stream>>>(
-        (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, block_table, table_stride,
-        (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, scale, window);
-  else
+  const bool terms = slopes != nullptr || soft_cap > 0.f;
+#define FMS_GEN(T, TERMS)                                                                                              \
+  attn_generic_kernel<T, TERMS><<<grid, GEN_THREADS, 0, stream>>>(                                                     \
+      (const T*)q, q_stride, (T*)out, out_stride, positions, seq_of_token, block_table, table_stride, (const T*)k_cache, \
+      (const T*)v_cache, nheads, kvheads, head_dim, scale, window, slopes, soft_cap)
+  if (dtype == FMS_F32) {
+    if (terms)
+      FMS_GEN(float, true);
+    else
+      FMS_GEN(float, false);
+  } else if (dtype == FMS_BF16) {
+    if (terms)
+      FMS_GEN(bf16, true);
+    else
+      FMS_GEN(bf16, false);
+  } else {
     FMS_REQUIRE(false, "attn_generic: unknown dtype %d", dtype);
+  }
+#undef FMS_GEN
   FMS_LAUNCH_CHECK("attn_generic");
   return 0;
 }

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define FMSAMD_ABI_VERSION 1
+#define FMSAMD_ABI_VERSION 2
 
 // element types
 #define FMS_F32 0
@@ -60,11 +60,13 @@ int fmsamd_rope_kv_write(void* qkv, int dtype, long row_stride, const int* posit
                          int rot_dim, int max_pos, void* k_cache, void* v_cache, int n_tokens, int nheads, int kvheads,
                          int head_dim, hipStream_t stream);
 
-// causal attention over the cache; any element type, any even head size up to 256
+// causal attention over the cache; any element type, any even head size up to 256.  Further terms of the scores:
+// slopes (float32 [nheads] or null): score += slopes[head] * (key position - query position); soft_cap (0: none):
+// score = soft_cap * tanh(score / soft_cap), before the slope term.
 int fmsamd_attn_generic(const void* q, long q_stride, void* out, long out_stride, int dtype, const int* positions,
                         const int* seq_of_token, const int* block_table, int table_stride, const void* k_cache,
                         const void* v_cache, int n_tokens, int nheads, int kvheads, int head_dim, float scale,
-                        int window, hipStream_t stream);
+                        int window, const float* slopes, float soft_cap, hipStream_t stream);
 
 // bfloat16 prefill: the step is cut into query blocks of at most fmsamd_attn_prefill_qblock(...) consecutive
 // tokens of one sequence; the same number goes into the call as qblock_tokens
@@ -155,6 +157,12 @@ int fmsamd_argmax(const float* logits, long ld, int rows, int vocab, void* works
 // The first call on a device looks the array's address up (hipGetSymbolAddress), so make it outside a capture.
 #define FMSAMD_ARGMAX_STATIC_BYTES (256 * 1024)
 int fmsamd_argmax_static(const float* logits, long ld, int rows, int vocab, int* out_tokens, hipStream_t stream);
+
+// Measurements of the GPU itself, for a benchmark's "of the measured peak": a pure read of `bytes` bytes by
+// `blocks` blocks, and blocks x 4 waves x iterations x 8 matrix instructions on registers (*flops: how many
+// floating-point operations that is).  `out` is a float on the device that may be written.
+int fmsamd_probe_read(const void* buffer, long bytes, int blocks, float* out, hipStream_t stream);
+int fmsamd_probe_mfma(int blocks, int iterations, float* out, double* flops, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -128,13 +128,15 @@ class DecodeGraph:
             rng = [[int(s), int(c)] for s, c in zip(seeds, counters)] + [[0, 0]] * pad
             self.rng.copy_(torch.tensor(rng, dtype=torch.int64), non_blocking=True)
         self.slots = tuple(slots)
-        self.n_pages = [pages_for(cache.length(s)) for s in slots]
+        self.n_pages = [(pages_for(cache.length(s)), cache.pages_held(s)) for s in slots]
 
     def refresh_pages(self) -> None:
-        """Write the block-table rows of sequences that got a new page since the last step."""
+        """Write the block-table rows of sequences that got a new page, or whose window gave one back, since the
+        last step: a page that was given back may be another sequence's by now, and its entry must read -1 in
+        the same step."""
         cache = self.engine.cache
         for row, slot in enumerate(self.slots):
-            n = pages_for(cache.length(slot))
+            n = (pages_for(cache.length(slot)), cache.pages_held(slot))
             if n != self.n_pages[row]:
                 for g, table in self.tables.items():
                     table[row].copy_(cache.block_table(g, [slot], n_columns=self.table_width)[0], non_blocking=True)

@@ -96,6 +96,10 @@ class Engine:
             return choose(logits, sampling, seeds, counters).tolist()
         if len(set(slots)) != len(slots) or len(tokens) != len(slots):
             raise ValueError("one token per sequence, each sequence once")
+        live = set(self.cache.live_slots())
+        for s in slots:
+            if s not in live:
+                raise ValueError(f"slot {s} is not live")
         for t in tokens:
             if not 0 <= t < self.vocab:
                 raise IndexError(f"token id {t} is outside the vocabulary of {self.vocab}")

@@ -8,7 +8,7 @@ from typing import List, Optional, Tuple
 import torch
 
 from ..cache import KVNeed, SequenceCache, StateNeed
-from ..parts import LayerCache, ModelSpec, Part, ResidualStream, make_part
+from ..parts import LayerCache, ModelSpec, Part, ResidualStream, make_part, part_attribute
 
 
 class DecoderModel(Part):
@@ -27,9 +27,14 @@ class DecoderModel(Part):
             pos = self.positions[layer.position] if layer.position is not None else None
             mixer = make_part("mixer", layer.mixer.kind, width=spec.width, position_encoder=pos, **layer.mixer.args)
             ff = make_part("feed_forward", layer.feed_forward.kind, width=spec.width, **layer.feed_forward.args)
-            norm1 = make_part("norm", layer.norm.kind, width=spec.width, **layer.norm.args)
-            norm2 = make_part("norm", layer.norm.kind, width=spec.width, **layer.norm.args)
-            block = make_part("block", layer.block.kind, mixer=mixer, feed_forward=ff, norm1=norm1, norm2=norm2, **layer.block.args)
+            # a block names the norms it wants as constructor arguments (none, two, four ...); each is built from the
+            # layer's list of norm specs, or from its one norm spec for all of them
+            wanted = part_attribute("block", layer.block.kind, "norm_arguments", ("norm1", "norm2"))
+            specs = layer.norms if layer.norms is not None else [layer.norm] * len(wanted)
+            if len(specs) != len(wanted):
+                raise ValueError(f"layer {i}: block {layer.block.kind!r} takes {len(wanted)} norms {tuple(wanted)}, {len(specs)} are given")
+            norms = {name: make_part("norm", n.kind, width=spec.width, **n.args) for name, n in zip(wanted, specs)}
+            block = make_part("block", layer.block.kind, mixer=mixer, feed_forward=ff, **norms, **layer.block.args)
             self.layers.append(self.add_child(spec.layer_name.format(i=i), block))
         self.final_norm = self.add_child(spec.final_norm_name, make_part("norm", spec.final_norm.kind, width=spec.width, **spec.final_norm.args))
         self.head = self.add_child(spec.head_name, make_part("head", spec.head.kind, width=spec.width, vocab=spec.vocab, **spec.head.args))
@@ -67,6 +72,43 @@ class DecoderModel(Part):
         for part in self.positions.values():
             part.finalize(self.device, self.dtype)
 
+    def state_dict(self, fused_weights: Optional[bool] = None) -> dict:
+        """Parameter names -> tensors, as the reference's model.state_dict() names them.  fused_weights (default: the
+        configuration's field): True gives the projections as the model holds them (qkv_fused, wg1_fused); False
+        gives the parts that the reference's unfused modules hold (fms/utils/fusion.py:15-35,
+        fms/modules/attention.py:666-687, fms/modules/feedforward.py:312-327): query/key/value and wg/w1, as views
+        of the fused tensors.  The model itself always runs the fused products; the field changes names at this
+        edge, and a checkpoint with either set of names loads (weights/adapters.py: weight_fusion)."""
+        if fused_weights is None:
+            fused_weights = bool(getattr(self.config, "fused_weights", True))
+        out = {}
+        for name, _, part, local in self.named_specs():
+            tensor = part.w[local]
+            if tensor is None:
+                target = self.tied.get(name)
+                tensor = out.get(target) if target else None
+            out[name] = tensor
+        if not fused_weights:
+            for part_name, part in self.named_parts():
+                for fused, pieces in getattr(part, "unfused_parameters", lambda: {})().items():
+                    for kind in ("weight", "bias"):
+                        whole = out.pop(f"{part_name}{fused}.{kind}", None)
+                        if whole is None:
+                            continue
+                        at = 0
+                        for piece, rows in pieces:
+                            out[f"{part_name}{piece}.{kind}"] = whole[at : at + rows]
+                            at += rows
+        return out
+
+    def named_parts(self, prefix: str = ""):
+        """(dotted name with a trailing dot, part) of every part below the model."""
+        stack = [(prefix, self)]
+        while stack:
+            name, part = stack.pop()
+            yield name, part
+            stack.extend((name + child_name + ".", child) for child_name, child in part.children().items())
+
     def get_config(self):
         """The configuration the model was built from (the reference's LLaMA.get_config, fms/models/llama.py:380-381)."""
         return self.config
@@ -82,7 +124,7 @@ class DecoderModel(Part):
     def forward(self, batch, cache: SequenceCache) -> torch.Tensor:
         """float32 logits [n wanted rows, vocab] of the tokens in `batch`; the cache is extended in place."""
         max_position = batch.max_context - 1
-        stream = ResidualStream(self.embedding.forward(batch.token_ids))
+        stream = ResidualStream(self.embedding.forward(batch.token_ids, batch))
         for n, entry in enumerate(self.schedule):
             block = self.layers[entry.layer]
             block.mixer.check_step(max_position)

@@ -17,7 +17,7 @@ import torch  # noqa: F401  (loads libamdhip64 before our library asks for it)
 
 from . import build as _build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _lib: Optional[ctypes.CDLL] = None
 _lock = threading.Lock()
@@ -33,7 +33,7 @@ _SIGNATURES = {
     "fmsamd_bias_add": [P, I, P, I, I, I, P],
     "fmsamd_rope_table": [P, P, P, I, I, P],
     "fmsamd_rope_kv_write": [P, I, L, P, P, P, I, P, P, I, I, P, P, I, I, I, I, P],
-    "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P],
+    "fmsamd_attn_generic": [P, L, P, L, I, P, P, P, I, P, P, I, I, I, I, F, I, P, F, P],
     "fmsamd_attn_prefill_bf16": [P, L, P, L, P, P, P, P, I, I, P, I, P, P, I, I, I, I, F, I, P],
     "fmsamd_attn_decode_bf16": [P, L, P, L, P, L, P, P, P, I, P, P, I, I, I, I, F, I, I, I, I, I, P, P],
     "fmsamd_qkv_rope_skinny_bf16": [P, L, P, P, I, P, L, I, I, P, P, P, I, P, P, I, I, P, P, I, I, I, P, P, L, P],
@@ -47,6 +47,8 @@ _SIGNATURES = {
     "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P, L, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
+    "fmsamd_probe_read": [P, L, I, P, P],
+    "fmsamd_probe_mfma": [I, I, P, P, P],
 }
 
 

@@ -337,8 +337,14 @@ def attention(
     force_generic: bool = False,
     staged: Optional[bool] = None,
     row_order: Optional[torch.Tensor] = None,
+    score_slopes: Optional[torch.Tensor] = None,
+    soft_cap: float = 0.0,
 ) -> torch.Tensor:
     """Causal attention of every token over the cache of its sequence -> [T, nheads*head_dim].
+
+    Further terms of the scores (a position encoding that acts on the scores, a capped attention): score_slopes,
+    float32 [nheads], adds slope[head] * (key position - query position); soft_cap c > 0 turns a score s into
+    c * tanh(s / c) first.  With either, both types run the generic kernel (the MFMA kernels have no such term).
 
     q is a [T, >= nheads*head_dim] view (the query columns of the qkv rows).  float32 runs the
     generic kernel; bfloat16 runs the MFMA kernels (prefill needs the query blocks, decode the
@@ -353,12 +359,19 @@ def attention(
     out = torch.empty(T, nheads * head_dim, dtype=q.dtype, device=q.device)
     lib = load()
     common_tail = (T, nheads, kvheads, head_dim, float(scale), int(window), _stream())
-    if q.dtype == torch.float32 or force_generic or head_dim % 16:
+    if score_slopes is not None:
+        _need_cuda(score_slopes)
+        if score_slopes.dtype != torch.float32 or tuple(score_slopes.shape) != (nheads,) or not score_slopes.is_contiguous():
+            raise ValueError(f"score_slopes must be a contiguous float32 [{nheads}] tensor")
+    if not (soft_cap >= 0.0 and math.isfinite(soft_cap)):
+        raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
+    if q.dtype == torch.float32 or force_generic or head_dim % 16 or score_slopes is not None or soft_cap > 0.0:
         for t0 in range(0, T, 65535):
             n = min(65535, T - t0)
             check(lib.fmsamd_attn_generic(q[t0:].data_ptr(), q.stride(0), out[t0:].data_ptr(), out.stride(0), _code(q.dtype),
                                           positions[t0:].data_ptr(), seq_of_token[t0:].data_ptr(), block_table.data_ptr(),
-                                          block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), n, *common_tail[1:]))
+                                          block_table.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), n, *common_tail[1:-1],
+                                          _ptr(score_slopes), float(soft_cap), common_tail[-1]))
         return out
     if decode:
         if max_context <= 0:
@@ -406,7 +419,9 @@ def decode_split(rows: int, n_pages: int):
     by_rows = min(-(-256 // max(rows, 1)), max(1, n_pages // 8))  # but no splits of under 8 pages: one for each wave
     splits = max(1, min(max(by_rows, -(-n_pages // 128)), n_pages))
     pages = -(-n_pages // splits)
-    waves = max(1, min(8 if rows * splits <= 512 else 4, pages))
+    import os
+    limit = int(os.environ.get("FMSAMD_EXP_W8", "512"))
+    waves = max(1, min(8 if rows * splits <= limit else 4, pages))
     return pages, waves
 
 
@@ -603,3 +618,31 @@ def sample(
     check(load().fmsamd_sample(logits.data_ptr(), logits.stride(0), rows, vocab, int(bool(do_sample)), float(temperature),
                                int(top_k or 0), _ptr(rng_state), out.data_ptr(), _stream()))
     return out
+
+
+# --------------------------------------------------------------------------
+def measured_peaks(read_mib: int = 1024, repeats: int = 5):
+    """(bytes per second of a pure read, bfloat16 matrix flops per second) as measured on this GPU now: the best of
+    `repeats` runs of a kernel that only reads a buffer of read_mib MiB, and of one that only issues matrix
+    instructions on registers.  Takes about a tenth of a second."""
+    lib = load()
+    buffer = torch.empty(read_mib << 20, dtype=torch.uint8, device="cuda").zero_()
+    out = torch.zeros(4, dtype=torch.float32, device="cuda")
+    flops = ctypes.c_double(0.0)
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best_ms(launch):
+        launch()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(repeats):
+            start.record()
+            launch()
+            end.record()
+            torch.cuda.synchronize()
+            best = min(best, start.elapsed_time(end))
+        return best
+
+    read_ms = best_ms(lambda: check(lib.fmsamd_probe_read(buffer.data_ptr(), buffer.numel(), 2048, out.data_ptr(), _stream())))
+    mfma_ms = best_ms(lambda: check(lib.fmsamd_probe_mfma(256 * 4, 512, out.data_ptr(), ctypes.byref(flops), _stream())))
+    return buffer.numel() / (read_ms / 1000), flops.value / (mfma_ms / 1000)

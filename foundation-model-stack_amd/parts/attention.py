@@ -40,6 +40,7 @@ class MultiHeadAttention(Mixer):
         position_encoder: Optional[PositionEncoding] = None,
         scale_factor: Optional[float] = None,
         window: int = 0,
+        soft_cap: float = 0.0,
     ):
         super().__init__()
         if kvheads <= 0 or nheads % kvheads:
@@ -49,10 +50,19 @@ class MultiHeadAttention(Mixer):
         self.width, self.nheads, self.kvheads, self.head_dim = width, nheads, kvheads, head_dim
         self.scale = float(scale_factor) if scale_factor is not None else 1.0 / math.sqrt(head_dim)
         self.window = int(window)
+        self.soft_cap = float(soft_cap)  # scores become soft_cap * tanh(score / soft_cap); 0: no cap
+        if self.soft_cap < 0:
+            raise ValueError(f"soft_cap {soft_cap} must be zero (none) or positive")
         self.position_encoder = position_encoder
         in_proj = self.add_child("in_proj", Part())
         self.qkv = in_proj.add_child("qkv_fused", Linear(width, (nheads + 2 * kvheads) * head_dim, use_bias))
         self.dense = self.add_child("dense", Linear(nheads * head_dim, width, use_bias))
+
+    def unfused_parameters(self) -> dict:
+        """The fused projection as the parts it is made of: fused local name -> ((local name, rows), ...), in the
+        order of the rows (fms/modules/attention.py:666-687)."""
+        H, K, D = self.nheads, self.kvheads, self.head_dim
+        return {"in_proj.qkv_fused": (("in_proj.query", H * D), ("in_proj.key", K * D), ("in_proj.value", K * D))}
 
     # ---- what the mixer asks of the cache ---------------------------------
     def kv_need(self) -> Optional[KVNeed]:
@@ -69,8 +79,11 @@ class MultiHeadAttention(Mixer):
         if self.position_encoder is not None:
             self.position_encoder.check_positions(max_position)
 
+    def _score_slopes(self) -> Optional[torch.Tensor]:
+        return self.position_encoder.score_slopes(self.nheads) if self.position_encoder is not None else None
+
     def prefill_qblock(self, n_tokens: int, dtype) -> int:
-        if dtype != torch.bfloat16 or self.head_dim % 16:
+        if dtype != torch.bfloat16 or self.head_dim % 16 or self.soft_cap > 0 or self._score_slopes() is not None:
             return 0  # the generic kernel takes tokens one by one
         return ops.prefill_qblock(self.nheads, self.kvheads, self.head_dim, n_tokens)
 
@@ -113,6 +126,7 @@ class MultiHeadAttention(Mixer):
             decode=batch.is_decode, max_context=batch.context_bound,
             qblock_start=qb_start, qblock_len=qb_len, qblock_tokens=size,
             row_order=batch.rows_by_length if batch.is_decode else None,
+            score_slopes=self._score_slopes(), soft_cap=self.soft_cap,
         )
         return BranchOutput(mixed, self.dense)
 

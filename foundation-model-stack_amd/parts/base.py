@@ -165,6 +165,16 @@ def list_parts(category: str) -> List[str]:
     return sorted(_registry[category])
 
 
+def part_attribute(category: str, kind: str, name: str, default=None):
+    """An attribute of the registered constructor (a class attribute of the part), or `default`: what a part says
+    about itself before it is built."""
+    try:
+        constructor = _registry[category][kind]
+    except KeyError:
+        raise KeyError(f"no {category} named {kind!r}; registered: {list_parts(category)}") from None
+    return getattr(constructor, name, default)
+
+
 def make_part(category: str, kind: str, **kwargs) -> Part:
     try:
         constructor = _registry[category][kind]

@@ -60,6 +60,7 @@ class ResidualStream:
 
 class PreNormBlock(Part):
     fuses_next_norm = True  # forward takes the norm that reads the stream after this block
+    norm_arguments = ("norm1", "norm2")  # the norms the block is built with, by constructor argument
 
     def __init__(self, mixer: Part, feed_forward: Part, norm1: Part, norm2: Part,
                  names=("ln", "attn", "ff_ln", "ff_sub_layer")):

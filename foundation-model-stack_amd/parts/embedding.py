@@ -18,8 +18,9 @@ class TokenEmbedding(Part):
         self.vocab, self.width = vocab, width
         self.declare("weight", (vocab, width))
 
-    def forward(self, token_ids: torch.Tensor) -> torch.Tensor:
-        """int32 ids [T] -> the float32 residual stream [T, width]."""
+    def forward(self, token_ids: torch.Tensor, batch=None) -> torch.Tensor:
+        """int32 ids [T] -> the float32 residual stream [T, width].  `batch` is the step (positions, sequence of
+        every token): an embedding that adds a learned vector per position reads it, this one does not."""
         return ops.embed(token_ids, self.w["weight"])
 
 

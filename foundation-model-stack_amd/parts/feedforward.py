@@ -24,6 +24,10 @@ class GatedLinearUnit(FeedForward):
         self.wg1 = self.add_child("wg1_fused", Linear(width, 2 * self.hidden_dim, use_bias))
         self.w2 = self.add_child("w2", Linear(self.hidden_dim, width, use_bias))
 
+    def unfused_parameters(self) -> dict:
+        """fms/modules/feedforward.py:312-327: the gate rows come first, then the "up" rows."""
+        return {"wg1_fused": (("wg", self.hidden_dim), ("w1", self.hidden_dim))}
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return self.forward_branch(x).value()
 

@@ -11,6 +11,9 @@ The interface a position encoding offers to a mixer:
     ``tables_for_step(batch)``: the same for one step, for encodings whose table depends on the step;
   * ``adjust_qk(qkv, batch, ...)``: transform queries and keys in place before
     they are cached, for encodings that are no plain rotation;
+  * ``score_slopes(nheads)``: for encodings that act on the scores instead (the reference's
+    ``adjusted_mask``, fms/modules/positions.py:9-36): a float32 slope per head, added to every score as
+    slope * (key position - query position); None for encodings that leave the scores alone;
   * ``check_positions(max_position)``: raise if a position cannot be encoded.
 """
 
@@ -68,6 +71,10 @@ class PositionEncoding(Part):
 
     def adjust_qk(self, qkv: torch.Tensor, batch, nheads: int, kvheads: int, head_dim: int) -> None:
         """In-place transform of the query and key columns of qkv rows; default: none."""
+
+    def score_slopes(self, nheads: int) -> Optional[torch.Tensor]:
+        """float32 [nheads] on the device: a bias by distance that attention adds to its scores; default: none."""
+        return None
 
     def check_positions(self, max_position: int) -> None:
         """Raise IndexError when `max_position` cannot be encoded."""

@@ -23,9 +23,10 @@ class PartSpec:
 class LayerSpec:
     mixer: PartSpec
     feed_forward: PartSpec
-    norm: PartSpec
+    norm: Optional[PartSpec] = None  # the spec of every norm the block asks for ...
     block: PartSpec = dataclasses.field(default_factory=lambda: PartSpec("pre_norm"))
     position: Optional[str] = None  # key into ModelSpec.positions, handed to the mixer
+    norms: Optional[List[PartSpec]] = None  # ... or one spec for each, in the order of the block's `norm_arguments`
 
 
 @dataclasses.dataclass

@@ -60,11 +60,12 @@ class Expected:
         return Expected._join(items, torch.cat)
 
 
-def expect(weights, cfg, ids, dtype) -> Expected:
-    exact = P.forward(weights, cfg, ids)
+def expect(weights, cfg, ids, dtype, **how) -> Expected:
+    """how: further arguments of the plain forward (calls=...: the sequence as it was fed, for ntk scaling)."""
+    exact = P.forward(weights, cfg, ids, **how)
     if dtype in ("float32", torch.float32):
         return Expected(exact)
-    reference = P.forward(weights, cfg, ids, storage=torch.bfloat16, rounding="reference")
+    reference = P.forward(weights, cfg, ids, storage=torch.bfloat16, rounding="reference", **how)
     error = (reference - exact).abs().amax(dim=-1)
     return Expected(exact, error, torch.quantile(error, 0.9).expand_as(error))
 

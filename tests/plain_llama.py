@@ -123,7 +123,8 @@ def rope_rotate(x: torch.Tensor, positions: torch.Tensor, freqs: torch.Tensor) -
     x is [S, heads, D]; pair i is (x[2i], x[2i+1]); angle = position * freqs[i];
     out[2i] = cos*x[2i] - sin*x[2i+1], out[2i+1] = sin*x[2i] + cos*x[2i+1].
     """
-    angles = torch.outer(positions.float(), freqs).float()  # [S, D/2]
+    # freqs [D/2], or [S, D/2] when the positions were rotated by different calls (ntk scaling with a cache)
+    angles = (torch.outer(positions.float(), freqs) if freqs.dim() == 1 else positions.float()[:, None] * freqs).float()
     cos = torch.cos(angles)[:, None, :]
     sin = torch.sin(angles)[:, None, :]
     pairs = x.float().reshape(*x.shape[:-1], -1, 2)
@@ -275,8 +276,15 @@ def forward(
     first_position: int = 0,
     storage=None,
     rounding: str = "stored",
+    calls: Optional[List[tuple]] = None,
 ) -> torch.Tensor:
     """fms/models/llama.py:137-162, 332-353, 444-445: logits [S, V] of one whole sequence.
+
+    calls (ntk scaling only): the sequence as a cache holds it after it was fed in several calls,
+    [(tokens of the call, longest sequence of the call's batch after it), ...].  fms/modules/positions.py:394-421:
+    a call rotates its queries and its new keys with the frequencies of alpha(max_start_pos + seq_len), and the
+    keys that earlier calls cached keep the rotation they got (fms/modules/attention.py:877-898: rotated before they
+    are stored).  Row p of the result is what the call that fed token p returned for it.
 
     storage=torch.bfloat16 sizes the error of running in bfloat16; `rounding` says where it rounds.
     "stored": every tensor that is stored between two operations (the outputs of norms, linears, rotation,
@@ -301,6 +309,11 @@ def forward(
         # tests/modules/test_positions.py:156-168: a position beyond the table raises
         raise IndexError("position beyond max_expected_seq_len")
     freqs = rope_frequencies(cfg.head_dim, cfg.theta, cfg.rope_scaling, int(positions[-1]) + 1, cfg.max_len)
+    if calls is not None:
+        if sum(n for n, _ in calls) != len(ids) or first_position:
+            raise ValueError("the calls must cover the sequence from its first token")
+        freqs = torch.cat([rope_frequencies(cfg.head_dim, cfg.theta, cfg.rope_scaling, longest, cfg.max_len)[None].expand(n, -1)
+                           for n, longest in calls])
     x = rs(embedding(w["base_model.embedding.weight"], tokens))
     for i in range(cfg.nlayers):
         p = f"base_model.layers.{i}."

@@ -241,6 +241,7 @@ def test_far_key_decides(lib, folders, dtype, tmp_path):
     cfg, weights = P.load_model_folder(folder)
     model = lib.get_model("hf_pretrained", model_path=folder, data_type=dtype)
     engine = Engine(model, max_tokens=1024, max_slots=1)
+    engine_two = Engine(model, max_tokens=2048, max_slots=2)
     ids = tokens_for("A", 700, 8)
     want = expect(weights, cfg, ids, dtype)
     # sharp indeed: the heaviest key of a late query holds most of its weight, and it lies far back
@@ -253,6 +254,28 @@ def test_far_key_decides(lib, folders, dtype, tmp_path):
         got.append(engine.step([slot], [[tok]], "last"))
     engine.end_sequence(slot)
     check(torch.cat(got), want, dtype, margin=SHARP_MARGIN)
+
+    # Negative controls: the same comparison has to fail when the cache loses one key, and when a step reads
+    # another sequence's slot.  The key that the late queries of the first layer lean on most is taken out.
+    heavy = int(torch.mode(probs.argmax(-1)).values)
+    assert heavy < 600
+    slot = engine.new_sequence()
+    engine.step([slot], [ids[:600]], "all")
+    for group in engine.cache.groups:
+        page = group.pages[slot][heavy // 64]
+        group.keys[:, page, :, heavy % 64, :] = 0
+        group.values[:, page, :, :, heavy % 64] = 0
+    lost = torch.cat([engine.step([slot], [[tok]], "last") for tok in ids[600:]])
+    engine.end_sequence(slot)
+    with pytest.raises(AssertionError):
+        check(lost, want[600:], dtype, margin=SHARP_MARGIN)
+    other = tokens_for("A", 600, 9)
+    a, b = engine_two.new_sequence(), engine_two.new_sequence()
+    engine_two.step([a, b], [ids[:600], other], "last")
+    swapped = torch.cat([engine_two.step([b, a], [[tok], [1]], "last")[:1] for tok in ids[600:640]])
+    with pytest.raises(AssertionError):
+        check(swapped, want[600:640], dtype, margin=SHARP_MARGIN)
+    engine.cache.check()
 
 
 # --------------------------------------------------------------------------
@@ -388,15 +411,19 @@ def test_bfloat16_generation_follows_the_plain_one(lib, folders):
     engine = Engine(get(lib, folders, name, "bfloat16"), max_tokens=1024, max_slots=8)
     prompts = [tokens_for(name, n, 40 + n) for n in (3, 30, 64, 65)]
     got = generate_requests(engine, prompts, max_new_tokens=12)
+    compared = total = 0
     for p, g in zip(prompts, got):
         ids = list(p)
         for tok in g:
             logits = P.forward(weights, cfg, ids)[-1]
             top = torch.topk(logits, 2).values
+            total += 1
             # where the plain logits separate the best token clearly, bfloat16 must pick it
             if float(top[0] - top[1]) > 0.05 * float(logits.abs().max()):
                 assert tok == int(logits.argmax())
+                compared += 1
             ids.append(tok)
+    assert total == 48 and compared >= total // 2, f"only {compared} of {total} tokens were compared"
     engine.cache.check()
 
 
@@ -803,6 +830,16 @@ def test_ntk_scaling(lib, dtype, tmp_path):
     assert engine.length(b) == 256
     with pytest.raises(IndexError):
         engine.step([b], [[1]], "last")
+    engine.end_sequence(b)
+    # a sequence that crosses both borders one token at a time: every step rotates its token with the alpha of its
+    # own length, and the keys in the cache keep the rotation of the step that wrote them (positions.py:394-421)
+    crossing = tokens_for("A", 140, 54)
+    c = engine.new_sequence()
+    got = [engine.step([c], [crossing[:60]], "all")] + [engine.step([c], [[t]], "last") for t in crossing[60:]]
+    calls = [(60, 60)] + [(1, n) for n in range(61, 141)]
+    check(torch.cat(got), expect(weights, cfg, crossing, dtype, calls=calls), dtype)
+    # and the same fed whole is another function: the plain forward tells the two apart by far more than the tolerance
+    assert float((P.forward(weights, cfg, crossing, calls=calls) - P.forward(weights, cfg, crossing))[60:].abs().max()) > 0.05
 
 
 @pytest.mark.parametrize("name", ["A", "C"])
@@ -865,9 +902,9 @@ def read_logits(out_dir, step, vocab):
     return torch.from_numpy(np.fromfile(os.path.join(out_dir, f"{step}.f32"), dtype="<f4").reshape(-1, vocab).copy())
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_trace_replay(lib, folders, dtype, tmp_path):
-    name = "A"
+def test_trace_replay(lib, folders, dtype, name, tmp_path):
     cfg, weights = plain(folders, name)
     V = cfg.vocab
     reqs = {"a": tokens_for(name, 100, 71), "b": tokens_for(name, 37, 72), "c": tokens_for(name, 70, 73),

@@ -380,6 +380,65 @@ def test_attention_over_long_contexts(ops):
     attention_case(ops, f32, 4, 2, 16, starts=[9000], lens=[1], decode=True)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_score_terms(ops, dtype):
+    """Further terms of the scores (fms/modules/positions.py:9-36, the reference's adjusted_mask; :78-105: a bias of
+    -|key position - query position| * scale[head]): a slope per head times the distance, and a soft cap.  Against
+    softmax(cap * tanh(q.k * scale / cap) - slope * distance) written out; the special cases: slope 0 and a cap far
+    above the scores is plain attention, a steep slope leaves every query its own value."""
+    torch.manual_seed(9)
+    H, K, D = 6, 2, 16
+    starts, lens = [0, 130, 5], [70, 2, 1]
+    totals = [s + n for s, n in zip(starts, lens)]
+    table, n_pages = make_pages(totals, K, D, dtype, seed=4)
+    ks = [torch.randn(n, K, D).to(dtype).float() for n in totals]
+    vs = [torch.randn(n, K, D).to(dtype).float() for n in totals]
+    qs = [2 * torch.randn(n, H, D).to(dtype).float() for n in lens]
+    kc, vc = fill_cache(table, ks, vs, n_pages, dtype)
+    q_flat = torch.cat([q.reshape(q.shape[0], H * D) for q in qs]).to(dtype)
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, lens)]).int()
+    seq = torch.cat([torch.full((n,), b) for b, n in enumerate(lens)]).int()
+    sc = 1 / math.sqrt(D)
+
+    def run(slopes, cap):
+        sl = dev(torch.tensor(slopes, dtype=torch.float32)) if slopes is not None else None
+        return ops.attention(dev(q_flat), dev(positions), dev(seq), dev(table), dev(kc), dev(vc), H, K, D, sc, 0,
+                             score_slopes=sl, soft_cap=cap, force_generic=True).cpu().float()
+
+    def want(slopes, cap):
+        outs = []
+        for q, k, v, s in zip(qs, ks, vs, starts):
+            n = q.shape[0]
+            pos = torch.arange(s, s + n)[:, None]
+            key = torch.arange(k.shape[0])[None, :]
+            o = torch.zeros(n, H, D)
+            for h in range(H):
+                kh = h // (H // K)
+                scores = (q[:, h].double() @ k[:, kh].double().t()) * sc
+                if cap:
+                    scores = cap * torch.tanh(scores / cap)
+                if slopes is not None:
+                    scores = scores - slopes[h] * (pos - key).abs()
+                probs = torch.softmax(scores.masked_fill(key > pos, float("-inf")), dim=-1)
+                o[:, h] = (probs @ v[:, kh].double()).float()
+            outs.append(o.reshape(n, H * D))
+        return torch.cat(outs)
+
+    tolerance = dict(atol=3e-5, rtol=3e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    slopes = [2.0 ** -(i + 1) for i in range(H)]
+    plain = run(None, 0.0)
+    torch.testing.assert_close(plain, want(None, 0.0), **tolerance)
+    for sl, cap in ((slopes, 0.0), (None, 1.5), (slopes, 1.5)):
+        got = run(sl, cap)
+        torch.testing.assert_close(got, want(sl, cap), **tolerance)
+        assert float((got - plain).abs().max()) > 0.05  # the term did something
+    torch.testing.assert_close(run([0.0] * H, 1e4), plain, **tolerance)
+    own = torch.cat([v[s : s + n].repeat_interleave(H // K, dim=1).reshape(n, H * D) for v, s, n in zip(vs, starts, lens)])
+    torch.testing.assert_close(run([200.0] * H, 0.0), own, **tolerance)
+    with pytest.raises(ValueError):
+        run(slopes[:-1], 0.0)
+
+
 def test_attention_generic_bf16_agrees(ops):
     attention_case(ops, torch.bfloat16, 4, 2, 16, starts=[0, 10], lens=[70, 3], force_generic=True)
 

@@ -306,6 +306,47 @@ def test_a_forced_type_casts_what_the_file_stores_in_32_bit(tmp_path):
     assert not kept.layers[0].mixer.dense.streams(4, torch.bfloat16)
 
 
+def test_state_dict_names_follow_fused_weights_and_load_back(tmp_path):
+    """tests/models/test_getmodel_fusedweights.py:30-33: a fused model's state dict has .qkv_fused. and .wg1_fused.,
+    an unfused one's .query./.key./.value. and .wg./.w1.; either loads into the model (fms/utils/fusion.py:15-35),
+    and so does a checkpoint with the names of before 0.0.6 (fms/models/llama.py:761-765)."""
+    config = LLaMAConfig(**TINY)
+    folder = fms_amd.write_model_folder(str(tmp_path / "m"), config, seed=4, data_type="float32")
+    model = DecoderModel(llama_spec(config), torch.float32, config=config)
+    load_checkpoint(model, folder, "llama", "hf", "cpu")
+    fused = model.state_dict()
+    assert any(".qkv_fused." in n for n in fused) and any(".wg1_fused." in n for n in fused)
+    assert not any(part in n for n in fused for part in (".query.", ".key.", ".value.", ".w1.", ".wg."))
+    model.config = config.updated(fused_weights=False)
+    unfused = model.state_dict()
+    assert not any(".qkv_fused." in n or ".wg1_fused." in n for n in unfused)
+    H, K, D, F = config.nheads, config.kv_heads, config.head_dim, config.ffn_hidden_dim
+    p = "base_model.layers.1."
+    q, k, v = (unfused[p + f"attn.in_proj.{w}.weight"] for w in ("query", "key", "value"))
+    assert q.shape[0] == H * D and k.shape[0] == K * D == v.shape[0]
+    assert torch.equal(torch.cat([q, k, v]), fused[p + "attn.in_proj.qkv_fused.weight"])
+    assert torch.equal(torch.cat([unfused[p + "ff_sub_layer.wg.weight"], unfused[p + "ff_sub_layer.w1.weight"]]),
+                       fused[p + "ff_sub_layer.wg1_fused.weight"])
+    assert unfused[p + "ff_sub_layer.wg.weight"].shape[0] == F
+    assert model.state_dict(fused_weights=True).keys() == fused.keys()
+
+    def reload(sd, name):
+        path = tmp_path / name
+        path.mkdir()
+        sd = {n: t.contiguous() for n, t in sd.items()}
+        write_safetensors(str(path / "model.safetensors"), [(n, tuple(t.shape), t.dtype) for n, t in sd.items()], lambda n: sd[n])
+        again = DecoderModel(llama_spec(config), torch.float32, config=config)
+        load_checkpoint(again, str(path), "llama", detect_source(list(sd)), "cpu")  # as get_model finds the source
+        for n, t in fused.items():
+            assert torch.equal(again.state_dict(fused_weights=True)[n], t), n
+
+    reload(fused, "fused")
+    reload(unfused, "unfused")
+    old_names = {n.replace(".attn.in_proj.", ".attn."): t for n, t in unfused.items()}
+    assert detect_source(list(old_names)) == "fms.pre0.0.6" and detect_source(list(unfused)) == "fms_unfused"
+    reload(old_names, "pre006")
+
+
 def test_the_architecture_tells_a_checkpoints_source():
     from fms_amd.architectures import get_architecture
 
@@ -480,6 +521,79 @@ def test_a_step_that_cannot_be_made_changes_nothing():
     assert again == a
     stamps.add(cache.stamp(again))
     assert len(stamps) == 3
+
+
+def test_a_graph_rewrites_its_table_when_a_window_gives_a_page_back():
+    """A windowed group gives a page back at a step that brings no new page.  The captured step's block table must
+    show -1 there in the same step: the page may be another sequence's by the next one."""
+    from types import SimpleNamespace
+
+    from fms_amd.engine.decode_graph import DecodeGraph
+    from fms_amd.sampling import SamplingParams
+
+    cache = make_cache(max_tokens=64 * 8, window=100)
+    engine = SimpleNamespace(device=torch.device("cpu"), cache=cache)
+    graph = DecodeGraph(engine, rows=2, max_context=2048, sampling=SamplingParams(do_sample=False))
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    cache.extend_many([a, b], [160, 10])
+    positions = cache.extend_many([a, b], [1, 1])
+    graph.load([a, b], [1, 2], positions, [0, 0], [0, 0])
+    windowed = 1
+    released_at = None
+    for step in range(40):
+        before = [len(g.pages[a]) for g in cache.groups]
+        cache.extend_many([a, b], [1, 1])
+        graph.refresh_pages()
+        for g in range(len(cache.groups)):
+            assert torch.equal(graph.tables[g][:2], cache.block_table(g, [a, b], n_columns=graph.table_width)), (step, g)
+        if released_at is None and cache.groups[windowed].pages[a][0] == -1:
+            released_at = step
+            assert [len(g.pages[a]) for g in cache.groups] == before  # no new page came with the release
+            assert int(graph.tables[windowed][0, 0]) == -1 and int(graph.tables[0][0, 0]) >= 0
+    assert released_at is not None
+    cache.check()
+
+
+def test_a_decode_step_on_an_ended_slot_is_refused_like_any_step():
+    from fms_amd.engine import Engine
+    from fms_amd.sampling import SamplingParams
+
+    cache = make_cache()
+    engine = object.__new__(Engine)
+    engine.cache, engine.vocab, engine.use_graphs = cache, 100, True
+    a, b = cache.alloc_slot(), cache.alloc_slot()
+    cache.extend_many([a, b], [3, 3])
+    cache.free_slot(b)
+    greedy = SamplingParams(do_sample=False)
+    with pytest.raises(ValueError, match="not live"):
+        engine.decode_and_choose([a, b], [1, 2], greedy)
+    with pytest.raises(ValueError, match="not live"):
+        engine.decode_and_choose([7], [1], greedy)
+    with pytest.raises(ValueError):
+        engine.decode_and_choose([a, a], [1, 2], greedy)
+    with pytest.raises(ValueError, match="not live"):
+        cache.stamp(b)
+    assert cache.length(a) == 3  # nothing grew
+    cache.check()
+
+
+def test_a_windows_releases_are_found_without_walking_the_sequence():
+    """The pages a window gives back are looked for from the first page still held: the plan of a step touches as
+    many list entries as it releases, however long the sequence is."""
+    cache = SequenceCache([(0, KVNeed(2, 16, 128))], [], 64 * 40, 2, 100_000, device=None)
+    s = cache.alloc_slot()
+    cache.extend(s, 64 * 30)
+    group = cache.groups[0]
+    assert group.first_held[s] == 0 and cache.pages_held(s) == 30
+    cache.extend(s, 1)  # the first query of this step is position 1920: keys before 1793 are out of sight
+    assert group.first_held[s] == 28 and group.pages[s][:28] == [-1] * 28 and cache.pages_held(s) == 3
+    for _ in range(200):
+        (_, release, _), = cache._plan(s, 1)
+        assert len(release) <= 1 and all(i >= group.first_held[s] for i in release)
+        cache.extend(s, 1)
+        cache.check()
+    cache.free_slot(s)
+    assert group.pool.n_free == 40 and s not in group.first_held
 
 
 def test_block_table_rows_follow_the_step_order():

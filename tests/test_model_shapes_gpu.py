@@ -275,3 +275,123 @@ def test_thirty_two_layers(deep, dtype):
         engine.end_sequence(slot)
         check(torch.cat(parts), expect(deep.weights, deep.cfg, s, dtype), dtype)
     engine.cache.check()
+
+
+# ---- the benchmark's context ---------------------------------------------------------------------------------------
+LONG = dict(SHAPES["llama3_8b_layers"], nlayers=1, max_expected_seq_len=8192)
+
+
+class LongShape(Shape):
+    """One layer of the Llama-3-8B shape with positions up to 8192.  The plain implementation's answers for the
+    two long sequences are worked out once and shared by the tests (a request that is the beginning of a longer one
+    has the longer one's first rows: causality)."""
+
+    def __init__(self, name, folder, lib):
+        super().__init__(name, folder, lib)
+        self.long_ids = self.tokens(8150, 1)
+        self.other_ids = self.tokens(3000, 2)
+        self._wanted = {}
+
+    def want(self, which, dtype):
+        if (which, dtype) not in self._wanted:
+            print(f"[long] plain implementation: {which} in {dtype}", flush=True)
+            self._wanted[(which, dtype)] = expect(self.weights, self.cfg, self.long_ids if which == "long" else self.other_ids, dtype)
+        return self._wanted[(which, dtype)]
+
+
+@pytest.fixture(scope="module")
+def long_shape(tmp_path_factory):
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    import fms_amd
+    from fms_amd.kernels import load
+
+    load()
+    folder = str(tmp_path_factory.mktemp("long"))
+    fms_amd.write_model_folder(folder, fms_amd.LLaMAConfig(**LONG), seed=29, std=0.02, norm_std=0.1)
+    s = LongShape("long", folder, fms_amd)
+    yield s
+    s.models.clear()
+    s._wanted.clear()
+    del s
+    gc.collect()
+    torch.cuda.empty_cache()
+
+
+def _decode(engine, slots, fed, dtype):
+    """The logits of one decode step: bfloat16 as generation runs it (a replayed graph, fed the given tokens whatever
+    it chose before), float32 as an eager step."""
+    if dtype == "bfloat16":
+        from fms_amd.sampling import SamplingParams
+
+        engine.decode_and_choose(slots, fed, SamplingParams(do_sample=False))
+        return engine.last_graph.logits[: len(slots)].clone()
+    return engine.step(slots, [[t] for t in fed], "last")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_context_of_8192_whole_and_last_32_one_by_one(long_shape, dtype):
+    """A request that fills the benchmark's context (8150 of 8192 positions), whole and with its last 32 tokens one by
+    one: 128 pages a sequence, the decode attention's split at that bound, the graph captured for a context of 8192."""
+    from fms_amd.engine import Engine
+
+    ids, want = long_shape.long_ids, long_shape.want("long", dtype)
+    engine = Engine(long_shape.model(dtype), max_tokens=8192, max_slots=1, use_graphs=dtype == "bfloat16")
+    slot = engine.new_sequence()
+    check(engine.step([slot], [ids], "all"), want, dtype)
+    engine.end_sequence(slot)
+    slot = engine.new_sequence()
+    rows = sorted(set(range(0, len(ids) - 32, 29)) | set(range(len(ids) - 96, len(ids) - 32)))
+    got = [engine.step([slot], [ids[:-32]], [rows])]
+    for tok in ids[-32:]:
+        got.append(_decode(engine, [slot], [tok], dtype))
+    engine.end_sequence(slot)
+    check(torch.cat(got), want[rows + list(range(len(ids) - 32, len(ids)))], dtype)
+    if dtype == "bfloat16":
+        assert engine.graph_captures == [(1, 8192)]
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_context_of_8192_in_a_ragged_batch_with_reused_slots(long_shape, dtype):
+    """Requests of 8000, 130 and 3000 tokens start together; the short one ends first, then the middle one; a second
+    batch takes their slots and pages."""
+    from fms_amd.engine import Engine
+
+    engine = Engine(long_shape.model(dtype), max_tokens=(125 + 3 + 47) * 64, max_slots=3, use_graphs=dtype == "bfloat16")
+    first = [  # (ids, prompt length, expected)
+        (long_shape.long_ids[:8000], 7990, long_shape.want("long", dtype)[:8000]),
+        (long_shape.tokens(130, 3), 127, None),
+        (long_shape.other_ids, 2993, long_shape.want("other", dtype)),
+    ]
+    second = [(long_shape.tokens(300, 4), 296, None), (long_shape.tokens(70, 5), 64, None), (long_shape.tokens(9, 6), 1, None)]
+    for requests in (first, second):
+        seqs = [dict(ids=ids, at=n, slot=engine.new_sequence(), want=w, got=[]) for ids, n, w in requests]
+        # of the prompts: the last 64 rows and some hundred spread ones
+        rows = [sorted(set(range(0, s["at"], 41)) | set(range(max(0, s["at"] - 64), s["at"]))) for s in seqs]
+        logits = engine.step([s["slot"] for s in seqs], [s["ids"][: s["at"]] for s in seqs], rows)
+        at = 0
+        for s, r in zip(seqs, rows):
+            s["rows"] = list(r)
+            s["got"].append(logits[at : at + len(r)])
+            at += len(r)
+        alive = list(seqs)
+        while True:
+            for s in alive:
+                if s["at"] == len(s["ids"]):
+                    engine.end_sequence(s["slot"])
+            alive = [s for s in alive if s["at"] < len(s["ids"])]
+            if not alive:
+                break
+            logits = _decode(engine, [s["slot"] for s in alive], [s["ids"][s["at"]] for s in alive], dtype)
+            for i, s in enumerate(alive):
+                s["got"].append(logits[i : i + 1])
+                s["rows"].append(s["at"])
+                s["at"] += 1
+        engine.cache.check()
+        assert engine.cache.live_slots() == []
+        for s in seqs:
+            want = s["want"] if s["want"] is not None else expect(long_shape.weights, long_shape.cfg, s["ids"], dtype)
+            check(torch.cat(s["got"]), want[s["rows"]], dtype)
+    if dtype == "bfloat16":
+        assert (4, 8192) in engine.graph_captures  # three sequences in a step of four rows, the bound of the long one

@@ -523,3 +523,146 @@ def test_a_toy_feed_forward_with_routing_and_a_toy_position_encoding(lib):
     finally:
         unregister_part("feed_forward", "routed")
         unregister_part("position", "distance_damping")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_toy_parts_at_three_seams(lib, dtype):
+    """Three more parts the library has never heard of, defined here and put together through the registries:
+      * an embedding that adds a learned vector per position (it reads the step's positions: the model hands every
+        embedding the batch);
+      * a position encoding that acts on the scores and not on queries and keys (a slope per head times the
+        distance, the reference's adjusted_mask seam, fms/modules/positions.py:9-36), with an attention whose
+        scores are capped;
+      * a block that wants four norms, before and after each branch, and says so.
+    Stepped by the engine (prompts whole, then token by token, unequal lengths, a reused slot) against a plain
+    computation; bfloat16 against float32 on the same rounded weights."""
+    from fms_amd.engine import Engine
+    from fms_amd.engine.model import DecoderModel
+    from fms_amd.kernels import ops
+    from fms_amd.parts import LayerSpec, ModelSpec, Part, PartSpec, register_part, unregister_part
+    from fms_amd.parts.position import PositionEncoding
+    from fms_amd.weights import init_random
+
+    V, E, H, K, D, HID, MAXLEN, CAP = 61, 48, 4, 2, 16, 80, 96, 3.0
+
+    class PositionedEmbedding(Part):
+        def __init__(self, vocab, width, max_len):
+            super().__init__()
+            self.declare("weight", (vocab, width))
+            self.declare("positions", (max_len, width))
+
+        def forward(self, token_ids, batch=None):
+            return ops.embed(token_ids, self.w["weight"]) + ops.embed(batch.positions, self.w["positions"])
+
+    class DistanceSlopes(PositionEncoding):
+        def __init__(self, steepest):
+            super().__init__()
+            self.steepest, self._slopes = float(steepest), {}
+
+        def slope_values(self, nheads):
+            return [self.steepest * 2.0 ** -h for h in range(nheads)]
+
+        def score_slopes(self, nheads):
+            if nheads not in self._slopes:
+                self._slopes[nheads] = torch.tensor(self.slope_values(nheads), dtype=torch.float32, device=DEV)
+            return self._slopes[nheads]
+
+    class SandwichBlock(Part):
+        norm_arguments = ("before_mixer", "after_mixer", "before_ff", "after_ff")
+
+        def __init__(self, mixer, feed_forward, before_mixer, after_mixer, before_ff, after_ff):
+            super().__init__()
+            self.mixer = self.add_child("attn", mixer)
+            self.feed_forward = self.add_child("ff_sub_layer", feed_forward)
+            self.norms = [self.add_child(n, p) for n, p in zip(("ln", "post_attn_ln", "ff_ln", "post_ff_ln"),
+                                                                (before_mixer, after_mixer, before_ff, after_ff))]
+
+        def forward(self, stream, batch, cache, act_dtype, next_norm=None):
+            h = stream.normed(self.norms[0], act_dtype)
+            out = self.mixer.forward(h, batch, cache)
+            zeros = torch.zeros(out.shape, dtype=torch.float32, device=out.device)
+            stream.add_branch(self.norms[1].add_norm(zeros, out, act_dtype))  # the branch's output through a norm of its own
+            h = stream.normed(self.norms[2], act_dtype)
+            out = self.feed_forward.forward(h)
+            zeros = torch.zeros(out.shape, dtype=torch.float32, device=out.device)
+            stream.add_branch(self.norms[3].add_norm(zeros, out, act_dtype))
+
+    def spec():
+        norms = [PartSpec("rmsnorm", {"eps": e}) for e in (1e-5, 1e-6, 1e-5, 1e-4)]
+        layer = LayerSpec(mixer=PartSpec("attention", {"nheads": H, "kvheads": K, "head_dim": D, "soft_cap": CAP}),
+                          feed_forward=PartSpec("glu", {"hidden_dim": HID, "activation": "gelu"}), norms=norms,
+                          block=PartSpec("sandwich"), position="slopes")
+        return ModelSpec(vocab=V, width=E, max_seq_len=MAXLEN, layers=[layer, layer], final_norm=PartSpec("rmsnorm", {"eps": 1e-5}),
+                         embedding=PartSpec("positioned", {"max_len": MAXLEN}),
+                         positions={"slopes": PartSpec("distance_slopes", {"steepest": 0.5})})
+
+    register_part("embedding", "positioned", PositionedEmbedding)
+    register_part("position", "distance_slopes", DistanceSlopes)
+    register_part("block", "sandwich", SandwichBlock)
+    try:
+        with pytest.raises(ValueError, match="takes 4 norms"):
+            bad = spec()
+            bad.layers[0].norms = bad.layers[0].norms[:2]
+            DecoderModel(bad, torch.float32)
+        model = DecoderModel(spec(), dtype)
+        init_random(model, 6, torch.device(DEV), std=0.25, norm_std=0.2)
+        model.finalize_all(DEV)
+        assert len(model.layers[0].norms) == 4 and model.layers[1].norms[3].eps == 1e-4
+        engine = Engine(model, max_tokens=256, max_slots=2)
+        w = {name: owner.w[local].float().cpu() for name, _, owner, local in model.named_specs()}
+        slopes = torch.tensor(DistanceSlopes(0.5).slope_values(H))
+
+        def plain(ids):
+            S = len(ids)
+            x = w["base_model.embedding.weight"][torch.tensor(ids)] + w["base_model.embedding.positions"][:S]
+            dist = (torch.arange(S)[:, None] - torch.arange(S)[None, :]).float()
+            for layer in (0, 1):
+                p = f"base_model.layers.{layer}."
+                h = P.rms_norm(x, w[p + "ln.weight"], 1e-5)
+                q, k, v = torch.split(h @ w[p + "attn.in_proj.qkv_fused.weight"].t(), [H * D, K * D, K * D], dim=-1)
+                q, k, v = q.reshape(S, H, D), k.reshape(S, K, D), v.reshape(S, K, D)
+                k, v = k.repeat_interleave(H // K, dim=1), v.repeat_interleave(H // K, dim=1)
+                scores = CAP * torch.tanh(torch.einsum("ihd,jhd->hij", q, k) / math.sqrt(D) / CAP) - slopes[:, None, None] * dist.abs()
+                probs = torch.softmax(scores.masked_fill(dist < 0, float("-inf")), -1)
+                mixed = torch.einsum("hij,jhd->ihd", probs, v).reshape(S, H * D) @ w[p + "attn.dense.weight"].t()
+                x = x + P.rms_norm(mixed, w[p + "post_attn_ln.weight"], 1e-6)
+                h = P.rms_norm(x, w[p + "ff_ln.weight"], 1e-5)
+                y = P.gated_feed_forward(h, w[p + "ff_sub_layer.wg1_fused.weight"], w[p + "ff_sub_layer.w2.weight"], act_name="gelu")
+                x = x + P.rms_norm(y, w[p + "post_ff_ln.weight"], 1e-4)
+            return P.rms_norm(x, w["base_model.dec_norm.weight"], 1e-5) @ w["head.weight"].t()
+
+        g = torch.Generator().manual_seed(3)
+        for lengths in ((70, 9), (33,)):  # the second round takes a slot of the first
+            seqs = [torch.randint(0, V, (n,), generator=g).tolist() for n in lengths]
+            slots = [engine.new_sequence() for _ in seqs]
+            logits = engine.step(slots, [s[:-3] for s in seqs], "all")
+            got, at = [], 0
+            for s in seqs:
+                got.append([logits[at : at + len(s) - 3]])
+                at += len(s) - 3
+            for i in range(3, 0, -1):
+                logits = engine.step(slots, [[s[-i]] for s in seqs], "last")
+                for b in range(len(seqs)):
+                    got[b].append(logits[b : b + 1])
+            for slot in slots:
+                engine.end_sequence(slot)
+            for ids, rows in zip(seqs, got):
+                close(torch.cat(rows).cpu(), plain(ids), dtype)
+        engine.cache.check()
+        # each of the three did something: the plain computation without it is far from the engine's logits
+        ids = torch.randint(0, V, (40,), generator=g).tolist()
+        slot = engine.new_sequence()
+        have = engine.step([slot], [ids], "all").cpu()
+        engine.end_sequence(slot)
+        full = plain(ids)
+        close(have, full, dtype)
+        w_keep = dict(w)
+        w["base_model.embedding.positions"] = torch.zeros_like(w["base_model.embedding.positions"])
+        assert float((plain(ids) - full).abs().max()) > 0.1 * float(full.abs().max())
+        w.update(w_keep)
+        slopes = slopes * 0
+        assert float((plain(ids) - full).abs().max()) > 0.02 * float(full.abs().max())
+    finally:
+        unregister_part("embedding", "positioned")
+        unregister_part("position", "distance_slopes")
+        unregister_part("block", "sandwich")

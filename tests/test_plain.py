@@ -206,6 +206,134 @@ def test_rope_llama3_scaling_limits():
     assert mid.any() and bool(((scaled[mid] < base[mid]) & (scaled[mid] > base[mid] / 8)).all())
 
 
+def _llama3_checks(freq_fn):
+    """What fixes the mid band of the llama3 scaling beside the reference's lines (fms/modules/positions.py:171-196).
+    Returns the list of checks that `freq_fn(dim, theta, scaling)` fails."""
+    failed = []
+    # 1. two frequencies worked out by hand.  D=16, theta=1e4: f_i = 1e4^(-i/8) = 1, 0.3162.., 0.1, 0.03162.., ...;
+    # original length 64, low 1, high 4, factor 8: wavelengths 6.28 (kept), 19.87 and 62.83 (between 64/4 and
+    # 64/1: interpolated), 198.7 and longer (divided by 8).  For i=1: smooth = (64/19.869.. - 1)/3 = 0.74035..,
+    # f = 0.25964..*0.31622../8 + 0.74035..*0.31622.. = 0.244384..; for i=2: smooth = 0.0061972.., f = 0.0130422..
+    small = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+             "original_max_position_embeddings": 64}
+    got = freq_fn(16, 10000.0, small)
+    by_hand = torch.tensor([1.0, 0.24438459943539834, 0.013042256043820465, 0.03162277660168379 / 8, 0.01 / 8])
+    if not torch.allclose(got[:5], by_hand, rtol=2e-5, atol=0):
+        failed.append("hand-computed vector")
+    # 2. the band as a whole, on many frequencies (D=1024 puts some hundred of them into it): scaled / unscaled is a
+    # straight line in 1/wavelength through (low edge, 1/factor) and (high edge, 1): continuous at both edges, and it
+    # rises with the frequency.
+    scaling = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0, "high_freq_factor": 4.0,
+               "original_max_position_embeddings": 8192}
+    base = freq_fn(1024, 500000.0, None).double()
+    ratio = freq_fn(1024, 500000.0, scaling).double() / base
+    per_length = base * 8192 / (2 * math.pi)  # original length / wavelength: 1 at the low edge, 4 at the high edge
+    mid = (per_length >= 1.0) & (per_length <= 4.0)
+    assert int(mid.sum()) > 50
+    line = 1 / 8 + (1 - 1 / 8) * (per_length - 1.0) / (4.0 - 1.0)
+    if not torch.allclose(ratio[mid], line[mid], rtol=1e-4, atol=0):
+        failed.append("line through the band's ends")
+    lowest, highest = ratio[mid][-1], ratio[mid][0]  # frequencies fall with the index
+    if not (abs(float(lowest) - 1 / 8) < 0.01 and abs(float(highest) - 1.0) < 0.02):
+        failed.append("continuity at the edges")
+    if not bool((ratio[mid][:-1] >= ratio[mid][1:]).all()):
+        failed.append("monotone")
+    if not (torch.equal(ratio[per_length > 4.0], torch.ones_like(ratio[per_length > 4.0]))
+            and torch.allclose(ratio[per_length < 1.0], torch.full_like(ratio[per_length < 1.0], 1 / 8), rtol=1e-6)):
+        failed.append("outside the band")
+    return failed
+
+
+def test_rope_llama3_mid_band():
+    """The interpolation between the kept and the divided frequencies (a Llama-3.1 config.json takes it)."""
+    assert _llama3_checks(lambda d, th, sc: P.rope_frequencies(d, th, sc)) == []
+
+
+def test_rope_llama3_checks_reject_plausible_mistakes():
+    """The checks above can fail: the interpolation weights swapped, the scaling left out, the band's ends swapped."""
+
+    def variant(kind):
+        def freqs(dim, theta, scaling):
+            f = 1.0 / (theta ** (torch.arange(0, dim, 2)[: dim // 2].float() / dim))
+            if not scaling or kind == "no scaling":
+                return f
+            factor, low, high = scaling["factor"], scaling["low_freq_factor"], scaling["high_freq_factor"]
+            old = scaling["original_max_position_embeddings"]
+            if kind == "ends swapped":
+                low, high = high, low
+            wavelen = 2 * math.pi / f
+            smooth = (old / wavelen - low) / (high - low)
+            if kind == "weights swapped":
+                smooth = 1 - smooth
+            out = torch.where(wavelen > old / min(low, high), f / factor, f)
+            band = (wavelen >= old / max(low, high)) & (wavelen <= old / min(low, high))
+            return torch.where(band, (1 - smooth) * f / factor + smooth * f, out)
+
+        return freqs
+
+    for kind in ("weights swapped", "no scaling", "ends swapped"):
+        failed = _llama3_checks(variant(kind))
+        assert "hand-computed vector" in failed and "line through the band's ends" in failed, (kind, failed)
+    assert _llama3_checks(variant("right")) == []
+
+
+def test_activations_are_the_library_functions():
+    """fms/utils/activation.py:6-24: every name is a torch.nn module; the formulas written out in the plain
+    implementation are those modules' functions."""
+    x = torch.linspace(-9, 9, 721)
+    x = torch.cat([x, torch.tensor([25.0, -25.0, 0.0])])  # mish's softplus is linear beyond 20
+    table = {
+        "gelu": F.gelu,
+        "gelu-tanh": lambda t: F.gelu(t, approximate="tanh"),
+        "gelu_pytorch_tanh": lambda t: F.gelu(t, approximate="tanh"),
+        "mish": F.mish,
+        "relu": F.relu,
+        "sigmoid": torch.sigmoid,
+        "silu": F.silu,
+        "swish": F.silu,
+        "tanh": torch.tanh,
+    }
+    for name, fn in table.items():
+        torch.testing.assert_close(P.activation(name)(x), fn(x), atol=1e-6, rtol=1e-5, msg=lambda m, n=name: f"{n}: {m}")
+        torch.testing.assert_close(P.activation(name.upper())(x), fn(x), atol=1e-6, rtol=1e-5)
+    # the two gelus differ by more than the tolerance, so a swapped pair fails the above
+    assert float((F.gelu(x) - F.gelu(x, approximate="tanh")).abs().max()) > 1e-4
+
+
+def test_ntk_scaling_keeps_the_rotation_of_cached_keys():
+    """fms/modules/positions.py:394-421 with a cache: every call rotates its new tokens with the frequencies of its
+    own alpha.  P.forward(calls=...) states that; here it is pinned by its special cases: calls within one alpha are
+    the whole-sequence forward, the last call's row depends on the alpha of earlier calls once a border was crossed,
+    and scores between tokens of one call still depend on their distance only."""
+    cfg = P.PlainConfig(vocab=50, width=24, nheads=3, kvheads=1, nlayers=2, hidden=40, eps=1e-5, theta=1e4, max_len=8,
+                        rope_scaling={"rope_type": "ntk", "factor": 4.0})
+    weights = {k: 8 * v for k, v in _fixture_weights(cfg, 12).items()}  # large enough for attention to choose
+    ids = [3, 9, 4, 4, 17, 30, 2, 8, 11, 12, 40, 41]
+    whole = P.forward(weights, cfg, ids)  # one call of 12 tokens: alpha 2 throughout
+    torch.testing.assert_close(P.forward(weights, cfg, ids, calls=[(12, 12)]), whole)
+    # fed in calls that all see alpha 2 (their batch's longest sequence has 9..16 tokens): the same logits
+    torch.testing.assert_close(P.forward(weights, cfg, ids, calls=[(5, 16), (4, 9), (3, 12)]), whole, atol=1e-5, rtol=1e-5)
+    # the first 8 tokens fed alone (alpha 1), the rest one by one (alpha 2): the first 8 rows are the regular model's,
+    # and the later rows differ from the whole call's, because they read keys rotated with the other base
+    stepped = P.forward(weights, cfg, ids, calls=[(8, 8), (1, 9), (1, 10), (1, 11), (1, 12)])
+    regular = P.PlainConfig(**{**cfg.__dict__, "rope_scaling": {}})
+    torch.testing.assert_close(stepped[:8], P.forward(weights, regular, ids[:8]), atol=1e-5, rtol=1e-5)
+    assert float((stepped[8:] - whole[8:]).abs().max()) > 1e-3
+    # the frequencies themselves: positions 0..7 those of alpha 1, 8..11 those of alpha 2 = theta * 2^(D/(D-2))
+    D = cfg.head_dim
+    f1 = P.rope_frequencies(D, cfg.theta)
+    f2 = P.rope_frequencies(D, cfg.theta * 2 ** (D / (D - 2)))
+    torch.testing.assert_close(P.rope_frequencies(D, cfg.theta, cfg.rope_scaling, 8, 8), f1)
+    torch.testing.assert_close(P.rope_frequencies(D, cfg.theta, cfg.rope_scaling, 9, 8), f2)
+    # a key of position 3 cached under alpha 1 against a query of position 9 under alpha 2: the score is the product
+    # of the two rotations, not a function of the distance
+    x = torch.randn(1, 1, D)
+    k3 = P.rope_rotate(x, torch.tensor([3]), f1)
+    q9 = P.rope_rotate(x, torch.tensor([9]), f2)
+    k3_same = P.rope_rotate(x, torch.tensor([3]), f2)
+    assert abs(float((q9 * k3).sum() - (q9 * k3_same).sum())) > 1e-3
+
+
 @pytest.mark.parametrize("H,K", [(4, 4), (4, 2), (4, 1), (1, 1)])
 def test_attention_is_library_attention(H, K):
     torch.manual_seed(5)

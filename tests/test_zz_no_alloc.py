@@ -38,15 +38,17 @@ def both(lib, logits):
     workspace = torch.empty(nbytes // 4, dtype=torch.float32, device="cuda")
     with_workspace = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
     without = torch.full((rows,), -1, dtype=torch.int32, device="cuda")
-    torch.cuda.synchronize()
-    before = torch.cuda.memory_allocated()
     code = lib.fmsamd_argmax(logits.data_ptr(), logits.stride(0), rows, vocab, workspace.data_ptr(), nbytes,
                              with_workspace.data_ptr(), stream)
     assert code == 0, lib.fmsamd_last_error().decode()
+    # Free device memory as the driver reports it (torch's own counters see torch's allocator only, and the entry
+    # point is called past it): nothing may be taken or given back between the two readings.
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
     code = lib.fmsamd_argmax_static(logits.data_ptr(), logits.stride(0), rows, vocab, without.data_ptr(), stream)
     assert code == 0, lib.fmsamd_last_error().decode()
     torch.cuda.synchronize()
-    assert torch.cuda.memory_allocated() == before
+    assert torch.cuda.mem_get_info()[0] == free_before
     return with_workspace.cpu(), without.cpu()
 
 
@@ -68,6 +70,35 @@ def test_two_calls_in_a_row_the_second_smaller(lib):
     wide = torch.randn(4, 9000, device="cuda")
     a, b = both(lib, wide[:, 1000:7000])
     assert a.tolist() == b.tolist() == wide[:, 1000:7000].argmax(-1).cpu().tolist()
+
+
+def test_the_call_can_be_captured_into_a_graph(lib):
+    """A stream that is capturing refuses every allocation on the host, without touching the GPU: after one call
+    that has looked the array's address up, the entry point records into a graph, and the replays (with the
+    program's own work between them) give what the eager call gives."""
+    torch.manual_seed(4)
+    logits = torch.randn(5, 40000, device="cuda")
+    out = torch.full((5,), -1, dtype=torch.int32, device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert lib.fmsamd_argmax_static(logits.data_ptr(), logits.stride(0), 5, 40000, out.data_ptr(), side.cuda_stream) == 0
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    assert out.tolist() == logits.argmax(-1).tolist()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        code = lib.fmsamd_argmax_static(logits.data_ptr(), logits.stride(0), 5, 40000, out.data_ptr(),
+                                        torch.cuda.current_stream().cuda_stream)
+    assert code == 0, lib.fmsamd_last_error().decode()
+    for replay in range(3):
+        logits.copy_(torch.randn(5, 40000, device="cuda"))
+        logits[replay, 123 + replay] = 30.0
+        out.fill_(-1)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert out.tolist() == logits.argmax(-1).tolist() and out[replay] == 123 + replay
 
 
 def test_sizes_beyond_the_scratch_array_are_refused(lib):
