@@ -92,6 +92,8 @@ __global__ void __launch_bounds__(GEN_THREADS)
 }
 
 #define LOG2E 1.4426950408889634f
+// the maximum that a partial result of the decode kernel carries when it holds no key at all
+#define DECODE_EMPTY -1e30f
 
 // Maxima as single instructions.  fmaxf() first passes each operand through a max with itself (it must quiet a
 // signalling NaN), which tripled the instructions of the score maxima; the scores here come out of the matrix unit
@@ -567,6 +569,243 @@ __global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_
 }
 
 // ==========================================================================
+// prefill through LDS with 32x32x16 products, for head sizes that are multiples of 32 up to 128.  The block is
+// that of attn_prefill_lds_kernel (four units of two waves, pages staged two at a time, fetched two ahead); a
+// wave's 32 query columns are one tile column.  On this GPU the 32x32x16 product runs at close to twice the
+// rate of the 16x16x32 one for the same operand bytes, and the prefill is bound by the matrix unit.
+//
+// S^T = K Q^T: a tile of 32 keys x 32 queries; lane (j = lane % 32, hb = lane / 32) holds query column j and
+// the 16 tile rows 8 (v / 4) + 4 hb + v % 4, v < 16.  Which key sits in which tile row is free: rows are dealt
+// so that those 16 are the keys 8 hb .. 8 hb + 7 (v < 8) and 16 + 8 hb .. 16 + 8 hb + 7 (v >= 8), each eight
+// the B operand of one step of O^T += V^T P^T, whose A operand is then one 16-byte read of a row of the
+// transposed value page.
+// ==========================================================================
+template <int DT32>
+struct WaveState32 {
+  f32x16 acc[DT32];  // O^T: d = dt * 32 + 8 (v / 4) + 4 hb + v % 4, query column j
+  float m, l;        // running maximum of the column (equal in its two lanes), this lane's share of the running sum
+};
+
+template <int DT32>
+__device__ __forceinline__ void half_step32(WaveState32<DT32>& st, const bf16x8 (&qreg)[DT32 * 2], int qpos, int qlo,
+                                            int key0, const bf16* kbase, int k_stride, const bf16* vbase, int v_stride,
+                                            float scale2, bool full) {
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int j = lane & 31, hb = lane >> 5;
+  // the key of tile row i = lane % 32 (this lane's row of the A operand): i = 8 blk + 4 h + e
+  const int key_row = 16 * (j >> 4) + 8 * ((j >> 2) & 1) + 4 * ((j >> 3) & 1) + (j & 3);
+  f32x16 sc;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+  {
+    bf16x8 ka[DT32 * 2];
+#pragma unroll
+    for (int c = 0; c < DT32 * 2; ++c) ka[c] = load_bf16x8(kbase + (size_t)key_row * k_stride + c * 16 + hb * 8);
+#pragma unroll
+    for (int c = 0; c < DT32 * 2; ++c) sc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[c], qreg[c], sc, 0, 0, 0);
+  }
+  if (!full) {
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+      const int key = key0 + 16 * (v >> 3) + 8 * hb + (v & 7);
+      sc[v] = (key <= qpos && key >= qlo) ? sc[v] : -INFINITY;
+    }
+  }
+  float mx = max3f(max3f(sc[0], sc[1], sc[2]), max3f(sc[3], sc[4], sc[5]), max3f(sc[6], sc[7], sc[8]));
+  mx = max3f(mx, max3f(sc[9], sc[10], sc[11]), max3f(sc[12], sc[13], max2f(sc[14], sc[15])));
+  {
+    const unsigned u = __float_as_uint(mx);
+    const auto halves = __builtin_amdgcn_permlane32_swap(u, u, false, false);  // the column's other lane
+    mx = max2f(__uint_as_float(halves[0]), __uint_as_float(halves[1]));
+  }
+  const float m_new = max2f(st.m, mx * scale2);  // the scale is positive: scaled once, after the maximum
+  const float alpha = __builtin_amdgcn_exp2f(st.m - m_new);
+  st.m = m_new;
+  float p[16], psum = 0.f;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    p[v] = __builtin_amdgcn_exp2f(fmaf(sc[v], scale2, -m_new));
+    psum += p[v];
+  }
+  st.l = st.l * alpha + psum;
+  bf16x8 pmat[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+    pmat[h] = bf16x8{(bf16)p[8 * h], (bf16)p[8 * h + 1], (bf16)p[8 * h + 2], (bf16)p[8 * h + 3],
+                     (bf16)p[8 * h + 4], (bf16)p[8 * h + 5], (bf16)p[8 * h + 6], (bf16)p[8 * h + 7]};
+  if (__any(alpha != 1.f)) {  // the running maximum seldom moves after the first keys
+#pragma unroll
+    for (int dt = 0; dt < DT32; ++dt) st.acc[dt] *= alpha;
+  }
+#pragma unroll
+  for (int dt = 0; dt < DT32; ++dt) {
+    bf16x8 va[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) va[h] = load_bf16x8(vbase + (size_t)(dt * 32 + j) * v_stride + 16 * h + 8 * hb);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) st.acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(va[h], pmat[h], st.acc[dt], 0, 0, 0);
+  }
+}
+
+template <int DT32, int UNITS>
+__global__ void __launch_bounds__(UNITS * 2 * WAVE) __attribute__((amdgpu_waves_per_eu(2, 2)))
+    attn_prefill_lds32_kernel(const bf16* __restrict__ q, long q_stride, bf16* __restrict__ out, long out_stride,
+                              const int* __restrict__ positions, const int* __restrict__ seq_of_token,
+                              const int* __restrict__ qblock_start, const int* __restrict__ qblock_len,
+                              int n_qblocks, const int* __restrict__ block_table, int table_stride,
+                              const bf16* __restrict__ k_cache, const bf16* __restrict__ v_cache, int nheads,
+                              int kvheads, float scale, int window, int hb) {
+  constexpr int head_dim = DT32 * 32;
+  constexpr int KS = head_dim + LDS_PAD;      // LDS row stride of the key page [64][KS]
+  constexpr int VS = PAGE_TOKENS + LDS_PAD;   // LDS row stride of the transposed value page [head_dim][VS]
+  constexpr int THREADS = UNITS * 2 * WAVE;
+  constexpr int k_chunks = PAGE_TOKENS * head_dim / 8;  // 16-byte chunks of a page and operand
+  constexpr int k_cols = head_dim / 8;
+  constexpr int CH = (k_chunks + THREADS - 1) / THREADS;
+  constexpr int K_ELEMS = PAGE_TOKENS * KS, V_ELEMS = head_dim * VS;
+  // at the end the same memory carries one wave's state to its partner: UNITS waves x 64 lanes x (DT32 * 16 + 2) floats
+  constexpr int MERGE_BYTES = UNITS * WAVE * (DT32 * 16 + 2) * 4;
+  constexpr int PAGE_ELEMS = K_ELEMS + V_ELEMS;
+  constexpr int STAGE_BYTES = 2 * PAGE_ELEMS * 2 > MERGE_BYTES ? 2 * PAGE_ELEMS * 2 : MERGE_BYTES;
+  __shared__ __attribute__((aligned(16))) unsigned char stage[STAGE_BYTES];
+  bf16* const ks = reinterpret_cast<bf16*>(stage);
+  bf16* const vs = ks + K_ELEMS;
+
+  // the longest blocks of a causal step go first (workgroups are handed out in linear order)
+  const int group = nheads / kvheads;
+  const int tiles = group / hb;
+  const int per_qb = kvheads * tiles;
+  const int qb = n_qblocks - 1 - (int)(blockIdx.x / per_qb);
+  const int y = blockIdx.x % per_qb;
+  const int kh = y / tiles;
+  const int wave = threadIdx.x / WAVE;
+  const int unit = wave % UNITS;   // which head and run of 32 query tokens
+  const int khalf = wave / UNITS;  // the two waves of a unit take the two halves (32 keys each) of every page
+  const int lane = threadIdx.x & (WAVE - 1);
+  const int j = lane & 31, hbit = lane >> 5;
+  const int h = kh * group + (y % tiles) * hb + unit % hb;
+  const int t_begin = qblock_start[qb];
+  const int t_end = t_begin + qblock_len[qb];
+  const int seq = seq_of_token[t_begin];
+  if (seq < 0) return;  // whole block: uniform
+  const int* bt = block_table + (size_t)seq * table_stride;
+  const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
+
+  // this wave's queries: column j is token t0 + j
+  const int t0 = t_begin + (unit / hb) * 32;
+  const bool has_work = t0 < t_end;
+  const int t = t0 + j;
+  const bool valid = t < t_end;
+  bf16x8 qreg[DT32 * 2];
+#pragma unroll
+  for (int c = 0; c < DT32 * 2; ++c) {
+    bf16x8 v = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (valid) v = load_bf16x8(q + (size_t)t * q_stride + (size_t)h * head_dim + c * 16 + hbit * 8);
+    qreg[c] = v;
+  }
+  const int qpos = valid ? positions[t] : -1;
+  const int qlo = (valid && window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+  int wave_hi = -1, wave_lo = 0, full_hi = -1, full_lo = 0;  // keys some / every column of the wave sees
+  if (has_work) {
+    const int t_last = (t0 + 32 < t_end ? t0 + 32 : t_end) - 1;
+    wave_hi = positions[t_last];
+    full_hi = positions[t0];
+    wave_lo = (window > 0 && full_hi - window + 1 > 0) ? full_hi - window + 1 : 0;
+    full_lo = (window > 0 && wave_hi - window + 1 > 0) ? wave_hi - window + 1 : 0;
+  }
+  const int blk_first = positions[t_begin];
+  const int blk_hi = positions[t_end - 1];
+  const int blk_lo = (window > 0 && blk_first - window + 1 > 0) ? blk_first - window + 1 : 0;
+  const int page_first = blk_lo / PAGE_TOKENS, page_last = blk_hi / PAGE_TOKENS;
+
+  constexpr int PF = 2;
+  bf16x8 kbuf[PF][CH], vbuf[PF][CH];
+  auto fetch = [&](int pi, bf16x8 (&kb)[CH], bf16x8 (&vb)[CH]) {
+    const size_t phys = readable_page(bt[pi]);
+    const bf16* kp = k_cache + phys * page_elems + (size_t)kh * PAGE_TOKENS * head_dim;
+    const bf16* vp = v_cache + phys * page_elems + (size_t)kh * head_dim * PAGE_TOKENS;
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int id = threadIdx.x + c * THREADS;
+      const size_t at = id < k_chunks ? (size_t)id * 8 : 0;  // the page is contiguous; never a load behind a branch
+      kb[c] = load_bf16x8(kp + at);
+      vb[c] = load_bf16x8(vp + at);
+    }
+  };
+  auto stash = [&](int which, const bf16x8 (&kb)[CH], const bf16x8 (&vb)[CH]) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int id = threadIdx.x + c * THREADS;
+      if (id < k_chunks) {
+        *reinterpret_cast<bf16x8*>(ks + which * PAGE_ELEMS + (id / k_cols) * KS + (id % k_cols) * 8) = kb[c];
+        *reinterpret_cast<bf16x8*>(vs + which * PAGE_ELEMS + (id / 8) * VS + (id % 8) * 8) = vb[c];
+      }
+    }
+  };
+
+  WaveState32<DT32> st;
+  st.m = -1e30f, st.l = 0.f;
+#pragma unroll
+  for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) st.acc[dt][v] = 0.f;
+
+  fetch(page_first, kbuf[0], vbuf[0]);
+  stash(0, kbuf[0], vbuf[0]);
+#pragma unroll
+  for (int d = 0; d < PF; ++d) fetch(page_first + 1 + d <= page_last ? page_first + 1 + d : page_last, kbuf[(1 + d) % PF], vbuf[(1 + d) % PF]);
+  block_sync_lds();  // not __syncthreads(): the pages under way must not be waited for
+  for (int p0 = page_first; p0 <= page_last; p0 += PF) {
+#pragma unroll
+    for (int d = 0; d < PF; ++d) {
+      const int pi = p0 + d;  // past the last page (the loop runs in steps of PF pages): nothing but the barrier
+      const int cur = d & 1;  // PF is even: the page's half of LDS
+      if (pi + 1 <= page_last) stash(cur ^ 1, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      fetch(pi + 1 + PF <= page_last ? pi + 1 + PF : page_last, kbuf[(d + 1) % PF], vbuf[(d + 1) % PF]);
+      const int key0 = pi * PAGE_TOKENS + khalf * 32;
+      if (has_work && pi <= page_last && !(key0 > wave_hi || key0 + 31 < wave_lo))  // uniform over the wave
+        half_step32<DT32>(st, qreg, qpos, qlo, key0, ks + cur * PAGE_ELEMS + khalf * 32 * KS, KS,
+                          vs + cur * PAGE_ELEMS + khalf * 32, VS, scale * LOG2E, key0 + 31 <= full_hi && key0 >= full_lo);
+      block_sync_lds();  // the page just multiplied is overwritten after the next one
+    }
+  }
+  __syncthreads();  // the loads still under way, before the memory changes its use
+
+  // ---- the two waves of a unit meet: the second hands its state over ----
+  float* const hand = reinterpret_cast<float*>(stage) + (size_t)(unit * WAVE + lane) * (DT32 * 16 + 2);
+  if (khalf == 1) {
+#pragma unroll
+    for (int dt = 0; dt < DT32; ++dt)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) hand[dt * 16 + v] = st.acc[dt][v];
+    hand[DT32 * 16] = st.m;
+    hand[DT32 * 16 + 1] = st.l;
+  }
+  __syncthreads();
+  if (khalf == 0 && has_work) {
+    const float m1 = hand[DT32 * 16], l1 = hand[DT32 * 16 + 1];
+    const float m = fmaxf(st.m, m1);
+    const float f0 = __builtin_amdgcn_exp2f(st.m - m), f1 = __builtin_amdgcn_exp2f(m1 - m);  // base-2 maxima
+    float l = st.l * f0 + l1 * f1;
+    l += __shfl_xor(l, 32, WAVE);
+    if (valid) {
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      bf16* orow = out + (size_t)t * out_stride + (size_t)h * head_dim;
+#pragma unroll
+      for (int dt = 0; dt < DT32; ++dt) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          const float* o1 = hand + dt * 16 + b * 4;
+          const bf16x4 o = {(bf16)((st.acc[dt][b * 4] * f0 + o1[0] * f1) * inv), (bf16)((st.acc[dt][b * 4 + 1] * f0 + o1[1] * f1) * inv),
+                            (bf16)((st.acc[dt][b * 4 + 2] * f0 + o1[2] * f1) * inv), (bf16)((st.acc[dt][b * 4 + 3] * f0 + o1[3] * f1) * inv)};
+          *reinterpret_cast<bf16x4*>(orow + dt * 32 + b * 8 + hbit * 4) = o;
+        }
+      }
+    }
+  }
+}
+
+// ==========================================================================
 // decode: one query token per sequence.  Grid (split, kv head x head tile,
 // token); the 16 columns of a wave's tiles are query heads that share the kv
 // head.  Every sequence deals its own pages out over the splits; the waves of
@@ -858,16 +1097,29 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
   const int seq = uniform_load(seq_of_token + t);
   const int cols = group - ht * tile_cols < tile_cols ? group - ht * tile_cols : tile_cols;  // query heads here
   const int head0 = kh * group + ht * tile_cols;
+  // A block without keys (a padding row, or a split beyond the sequence's pages) leaves a maximum that marks its
+  // partial result as empty: the merge kernel then needs no index data to tell which splits count.
+  auto leave_empty = [&]() {
+    if (n_splits > 1 && (int)threadIdx.x < cols) {
+      const size_t base = ((size_t)t * nheads + head0 + threadIdx.x) * n_splits + split;
+      part_ml[base * 2] = DECODE_EMPTY;
+      part_ml[base * 2 + 1] = 0.f;
+    }
+  };
   if (seq < 0) {
-    if (split == 0)
+    if (n_splits == 1)
       for (int i = threadIdx.x; i < cols * head_dim; i += blockDim.x)
         out[(size_t)t * out_stride + (size_t)head0 * head_dim + i] = (bf16)0.f;
+    leave_empty();
     return;
   }
   const int pos = uniform_load(positions + t);
   const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   int page_lo, page_hi;
-  if (split >= split_pages(lo, pos, n_splits, split, &page_lo, &page_hi)) return;
+  if (split >= split_pages(lo, pos, n_splits, split, &page_lo, &page_hi)) {
+    leave_empty();
+    return;
+  }
 
   const int* bt = block_table + (size_t)seq * table_stride;
   const size_t page_elems = (size_t)kvheads * PAGE_TOKENS * head_dim;
@@ -941,42 +1193,40 @@ __global__ void __launch_bounds__(MAXW* WAVE) __attribute__((amdgpu_waves_per_eu
 }
 
 // one block per (head, token): combine the partial results of the splits.  The loads of four splits are
-// issued together (a loop that loads, waits and combines split by split pays the memory's latency per split).
+// issued together (a loop that loads, waits and combines split by split pays the memory's latency per split),
+// and none of them waits for index data: a split without keys carries the maximum DECODE_EMPTY, and whatever
+// its other numbers are, they are set aside (a row of which every split is empty, a padding row, becomes zeros).
 __global__ void attn_decode_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                         bf16* __restrict__ out, long out_stride, const int* __restrict__ positions,
-                                         const int* __restrict__ seq_of_token, int nheads, int head_dim, int n_splits,
-                                         int window) {
+                                         bf16* __restrict__ out, long out_stride, int nheads, int head_dim, int n_splits) {
   const int h = blockIdx.x;
   const int t = blockIdx.y;
-  if (uniform_load(seq_of_token + t) < 0) return;  // the decode kernel wrote zeros
-  const int pos = uniform_load(positions + t);
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-  int page_lo, page_hi;
-  const int active = split_pages(lo, pos, n_splits, 0, &page_lo, &page_hi);
   const size_t base = ((size_t)t * nheads + h) * n_splits;
   for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float m = -1e30f, o = 0.f, l = 0.f;  // running maximum (a base-2 logarithm), sum of values, sum of weights
-    for (int s0 = 0; s0 < active; s0 += 4) {
+    float m = DECODE_EMPTY, o = 0.f, l = 0.f;  // running maximum (a base-2 logarithm), sum of values, sum of weights
+    for (int s0 = 0; s0 < n_splits; s0 += 4) {
       float ms[4], ls[4], os[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int s = s0 + i < active ? s0 + i : active - 1;  // past the end: the last split again, given no weight
+        const int s = s0 + i < n_splits ? s0 + i : n_splits - 1;  // past the end: the last split again, given no weight
         ms[i] = part_ml[(base + s) * 2];
         ls[i] = part_ml[(base + s) * 2 + 1];
         os[i] = part_o[(base + s) * head_dim + d];
       }
+      bool counts[4];
       float m_new = m;
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (s0 + i < active) m_new = fmaxf(m_new, ms[i]);
+      for (int i = 0; i < 4; ++i) {
+        counts[i] = s0 + i < n_splits && ms[i] > 0.5f * DECODE_EMPTY;
+        if (counts[i]) m_new = fmaxf(m_new, ms[i]);
+      }
       const float keep = __builtin_amdgcn_exp2f(m - m_new);
       o *= keep;
       l *= keep;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float f = s0 + i < active ? __builtin_amdgcn_exp2f(ms[i] - m_new) : 0.f;
-        o += f * os[i];
-        l += f * ls[i];
+        const float f = __builtin_amdgcn_exp2f(ms[i] - m_new);
+        o += counts[i] ? f * os[i] : 0.f;
+        l += counts[i] ? f * ls[i] : 0.f;
       }
       m = m_new;
     }
@@ -1096,10 +1346,19 @@ extern "C" int fmsamd_attn_prefill_bf16(const void* q, long q_stride, void* out,
       n_qblocks, block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, head_dim, \
       scale, window, hb);                                                                                          \
   } while (0)
-  if (head_dim <= 64)
+#define FMS_PL32(D32)                                                                                              \
+  attn_prefill_lds32_kernel<D32, LDS_UNITS><<<grid, dim3(LDS_UNITS * 2 * WAVE), 0, stream>>>(                      \
+      (const bf16*)q, q_stride, (bf16*)out, out_stride, positions, seq_of_token, qblock_start, qblock_len, n_qblocks, \
+      block_table, table_stride, (const bf16*)k_cache, (const bf16*)v_cache, nheads, kvheads, scale, window, hb)
+  if (head_dim == 128)  // head sizes with a 32x32x16 kernel of their own
+    FMS_PL32(4);
+  else if (head_dim == 64)
+    FMS_PL32(2);
+  else if (head_dim <= 64)
     FMS_PL(4);
   else
     FMS_PL(8);
+#undef FMS_PL32
 #undef FMS_PL
   FMS_LAUNCH_CHECK("attn_prefill_bf16");
   return 0;
@@ -1160,8 +1419,8 @@ extern "C" int fmsamd_attn_decode_bf16(const void* q, long q_stride, void* out, 
   FMS_LAUNCH_CHECK("attn_decode_bf16");
   if (n_splits > 1) {
     dim3 mgrid(nheads, n_tokens);
-    attn_decode_merge_kernel<<<mgrid, head_dim <= 64 ? 64 : 128, 0, stream>>>(
-        part_o, part_ml, (bf16*)out, out_stride, positions, seq_of_token, nheads, head_dim, n_splits, window);
+    attn_decode_merge_kernel<<<mgrid, head_dim <= 64 ? 64 : 128, 0, stream>>>(part_o, part_ml, (bf16*)out, out_stride, nheads,
+                                                                              head_dim, n_splits);
     FMS_LAUNCH_CHECK("attn_decode_merge");
   }
   return 0;

@@ -161,8 +161,10 @@ int fmsamd_argmax_static(const float* logits, long ld, int rows, int vocab, int*
 // Measurements of the GPU itself, for a benchmark's "of the measured peak": a pure read of `bytes` bytes by
 // `blocks` blocks, and blocks x 4 waves x iterations x 8 matrix instructions on registers (*flops: how many
 // floating-point operations that is).  `out` is a float on the device that may be written.
-int fmsamd_probe_read(const void* buffer, long bytes, int blocks, float* out, hipStream_t stream);
-int fmsamd_probe_mfma(int blocks, int iterations, float* out, double* flops, hipStream_t stream);
+// contiguous: every block reads one stretch of the buffer instead of the grid sweeping it together; large: 32x32x16
+// products instead of 16x16x32.
+int fmsamd_probe_read(const void* buffer, long bytes, int blocks, int contiguous, float* out, hipStream_t stream);
+int fmsamd_probe_mfma(int blocks, int iterations, int large, float* out, double* flops, hipStream_t stream);
 
 #ifdef __cplusplus
 }

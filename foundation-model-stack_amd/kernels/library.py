@@ -47,8 +47,8 @@ _SIGNATURES = {
     "fmsamd_gemm_skinny_residual_bf16": [P, L, P, P, I, P, L, P, I, P, L, P, I, I, I, I, P, P, L, P],
     "fmsamd_sample": [P, L, I, I, I, F, I, P, P, P],
     "fmsamd_argmax": [P, L, I, I, P, L, P, P],
-    "fmsamd_probe_read": [P, L, I, P, P],
-    "fmsamd_probe_mfma": [I, I, P, P, P],
+    "fmsamd_probe_read": [P, L, I, I, P, P],
+    "fmsamd_probe_mfma": [I, I, I, P, P, P],
 }
 
 

@@ -419,9 +419,7 @@ def decode_split(rows: int, n_pages: int):
     by_rows = min(-(-256 // max(rows, 1)), max(1, n_pages // 8))  # but no splits of under 8 pages: one for each wave
     splits = max(1, min(max(by_rows, -(-n_pages // 128)), n_pages))
     pages = -(-n_pages // splits)
-    import os
-    limit = int(os.environ.get("FMSAMD_EXP_W8", "512"))
-    waves = max(1, min(8 if rows * splits <= limit else 4, pages))
+    waves = max(1, min(8 if rows * splits <= 512 else 4, pages))
     return pages, waves
 
 
@@ -643,6 +641,12 @@ def measured_peaks(read_mib: int = 1024, repeats: int = 5):
             best = min(best, start.elapsed_time(end))
         return best
 
-    read_ms = best_ms(lambda: check(lib.fmsamd_probe_read(buffer.data_ptr(), buffer.numel(), 2048, out.data_ptr(), _stream())))
-    mfma_ms = best_ms(lambda: check(lib.fmsamd_probe_mfma(256 * 4, 512, out.data_ptr(), ctypes.byref(flops), _stream())))
-    return buffer.numel() / (read_ms / 1000), flops.value / (mfma_ms / 1000)
+    # the best of a few shapes of each: what the hardware can do, not what one launch shape happens to reach
+    read_ms = min(best_ms(lambda b=blocks, c=contiguous: check(lib.fmsamd_probe_read(buffer.data_ptr(), buffer.numel(), b, c, out.data_ptr(), _stream())))
+                  for blocks in (1024, 2048, 4096) for contiguous in (0, 1))
+    mfma = 0.0
+    for large in (0, 1):
+        for blocks in (256 * 2, 256 * 4):
+            ms = best_ms(lambda: check(lib.fmsamd_probe_mfma(blocks, 512, large, out.data_ptr(), ctypes.byref(flops), _stream())))
+            mfma = max(mfma, flops.value / (ms / 1000))
+    return buffer.numel() / (read_ms / 1000), mfma

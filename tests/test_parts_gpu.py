@@ -256,6 +256,117 @@ def test_a_toy_mixer_with_state_of_its_own(lib):
         unregister_part("mixer", "running_mean")
 
 
+def test_a_toy_mixer_whose_state_is_updated_on_the_device_under_capture(lib):
+    """The same running mean, with its state updated by device code that a graph can hold: the decode step finds each
+    row's state through the step's device-side index data (sequence of the row, slot of the sequence), padding rows add
+    nothing, and nothing is decided on the host.  The engine then replays decode steps as captured graphs; they give
+    what eager steps give and what the plain computation gives, over a batch that shrinks and slots that are reused."""
+    from fms_amd.cache import StateNeed
+    from fms_amd.engine import Engine
+    from fms_amd.engine.model import DecoderModel
+    from fms_amd.parts import LayerSpec, Mixer, ModelSpec, PartSpec, register_part, unregister_part
+    from fms_amd.sampling import SamplingParams
+    from fms_amd.weights import init_random
+
+    class RunningMeanOnDevice(Mixer):
+        def __init__(self, width, position_encoder=None):
+            super().__init__()
+            self.width = width
+            self.declare("proj.weight", (width, width))
+
+        def state_need(self):
+            return StateNeed((("sum", (self.width,), "float32"), ("count", (1,), "float32")))
+
+        def forward(self, x, batch, cache):
+            total, count = cache.state["sum"], cache.state["count"]
+            weight = self.w["proj.weight"].float()
+            if batch.is_decode:  # one row a sequence: index operations only, all on the device
+                live = batch.seq_of_token >= 0
+                slots = batch.slot_ids.long()[batch.seq_of_token.clamp(min=0).long()]
+                total.index_add_(0, slots, x.float() * live[:, None])
+                count.index_add_(0, slots, live.float()[:, None])
+                return ((total[slots] / count[slots].clamp(min=1.0)) @ weight.t()).to(x.dtype)
+            out = torch.empty_like(x)
+            at = 0
+            for slot, n in zip(batch.slots, batch.q_lens):  # a prompt: its rows one after another
+                sums = torch.cumsum(x[at : at + n].float(), 0) + total[slot]
+                counts = count[slot] + torch.arange(1, n + 1, device=x.device, dtype=torch.float32)
+                out[at : at + n] = ((sums / counts[:, None]) @ weight.t()).to(x.dtype)
+                total[slot] = sums[-1]
+                count[slot] += n
+                at += n
+            return out
+
+    V, E = 90, 48
+
+    def spec():
+        norm = PartSpec("rmsnorm", {"eps": 1e-5})
+        ff = PartSpec("glu", {"hidden_dim": 64, "activation": "swish"})
+        mean_layer = LayerSpec(mixer=PartSpec("running_mean_on_device"), feed_forward=ff, norm=norm)
+        attn_layer = LayerSpec(mixer=PartSpec("attention", {"nheads": 3, "kvheads": 1, "head_dim": 16}), feed_forward=ff,
+                               norm=norm, position="rope")
+        return ModelSpec(vocab=V, width=E, max_seq_len=256, layers=[mean_layer, attn_layer], final_norm=norm,
+                         positions={"rope": PartSpec("rope", {"dim": 16, "theta": 1e4, "max_seq_len": 256})})
+
+    register_part("mixer", "running_mean_on_device", RunningMeanOnDevice)
+    try:
+        model = DecoderModel(spec(), torch.float32)
+        init_random(model, 8, torch.device(DEV), std=0.2, norm_std=0.1)
+        model.finalize_all(DEV)
+        w = {name: owner.w[local].float().cpu() for name, _, owner, local in model.named_specs()}
+
+        def plain(ids):
+            x = w["base_model.embedding.weight"][torch.tensor(ids)]
+            cfg = P.PlainConfig(vocab=V, width=E, nheads=3, kvheads=1, nlayers=2, hidden=64, eps=1e-5, theta=1e4, max_len=256)
+            for layer in (0, 1):
+                p = f"base_model.layers.{layer}."
+                h = P.rms_norm(x, w[p + "ln.weight"], 1e-5)
+                if layer == 0:
+                    h = (torch.cumsum(h, 0) / torch.arange(1, len(ids) + 1)[:, None]) @ w[p + "attn.proj.weight"].t()
+                else:
+                    h = P.attention_block(h, torch.arange(len(ids)), cfg, w[p + "attn.in_proj.qkv_fused.weight"],
+                                          w[p + "attn.dense.weight"], P.rope_frequencies(16, 1e4))
+                x = x + h
+                h = P.rms_norm(x, w[p + "ff_ln.weight"], 1e-5)
+                x = x + P.gated_feed_forward(h, w[p + "ff_sub_layer.wg1_fused.weight"], w[p + "ff_sub_layer.w2.weight"])
+            return P.rms_norm(x, w["base_model.dec_norm.weight"], 1e-5) @ w["head.weight"].t()
+
+        greedy = SamplingParams(do_sample=False)
+        g = torch.Generator().manual_seed(5)
+        chosen = {}
+        for graphs in (True, False):
+            engine = Engine(model, max_tokens=512, max_slots=3, use_graphs=graphs)
+            assert engine.use_graphs == graphs  # nothing in the model refuses capture
+            g.manual_seed(5)
+            tokens_of_run = []
+            for round_ in range(2):  # the second round takes the slots again: their state starts at zero
+                prompts = [torch.randint(0, V, (n,), generator=g).tolist() for n in (20, 3, 9)]
+                slots = [engine.new_sequence() for _ in prompts]
+                first = engine.step(slots, prompts, "last").argmax(-1).tolist()
+                seqs = [p + [t] for p, t in zip(prompts, first)]
+                alive = [0, 1, 2]
+                for step in range(7):
+                    if step == 4:  # the middle sequence ends: the batch's rows change under the graph
+                        engine.end_sequence(slots[1])
+                        alive = [0, 2]
+                    new = engine.decode_and_choose([slots[b] for b in alive], [seqs[b][-1] for b in alive], greedy)
+                    logits = engine.last_graph.logits[: len(alive)].cpu() if graphs else None
+                    for i, b in enumerate(alive):
+                        if graphs:  # the logits of the fed token, against the plain computation of the sequence so far
+                            torch.testing.assert_close(logits[i], plain(seqs[b])[-1], atol=2e-4, rtol=1e-3)
+                        seqs[b].append(new[i])
+                for b in alive:
+                    engine.end_sequence(slots[b])
+                tokens_of_run.append(seqs)
+            if graphs:
+                assert len(engine.graph_captures) >= 2
+            engine.cache.check()
+            chosen[graphs] = tokens_of_run
+        assert chosen[True] == chosen[False]
+    finally:
+        unregister_part("mixer", "running_mean_on_device")
+
+
 def test_a_layer_named_twice_and_a_layer_reading_another_cache(lib, tmp_path):
     """The order of layers is data: Llama's own layers in the order 0, 1, 0, with the last entry
     reading the keys and values that the first one cached (it computes queries only)."""
