@@ -11,8 +11,6 @@
 //     sums meet in LDS.  Epilogues: plain, act(x Wg^T) * (x Wu^T), rotation
 //     and cache write, addition into the residual stream.  The entry points
 //     hand 17 to 128 rows to the kernels of gemm_wide.hip.
-#include <stdlib.h>
-
 #include "common.h"
 #include "fmsamd.h"
 #include "gemm_epilogue.h"
@@ -224,15 +222,12 @@ extern "C" int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const vo
 // SK_WAVES: waves of a block.
 // UNR: groups of 128 k-values whose loads a wave issues before it multiplies: what keeps enough
 // bytes in flight to stream from HBM (a wave has UNR * (NTB + MT) * 4 loads of 16 bytes outstanding).
-// XD: the rows of x are loaded straight into the MFMA operand layout (16 rows x 64 bytes an instruction) instead of
-// in long runs through LDS: x comes from L2, where the shape of a load matters little, and with several tiles of
-// x a wave the LDS traffic of their layout change would outweigh that of the weights.
-template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typename BiasT, bool XD = false>
+template <int SK_WAVES, int UNR, int NTB, int MT, int EPI, typename OutT, typename BiasT>
 __global__ void __launch_bounds__(SK_WAVES* WAVE)
     __attribute__((amdgpu_waves_per_eu(MT > 1 ? 2 : 4)))  // two blocks a compute unit; one with several tiles of x
     skinny_bf16_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, const BiasT* __restrict__ bias,
                        OutT* __restrict__ out, long ldo, int M, int N, int K, int tile2_offset, int act,
-                       int rows_per_block, RowScale scale, RopeEpilogue rope, ResidEpilogue res, int rotate) {
+                       int rows_per_block, RowScale scale, RopeEpilogue rope, ResidEpilogue res) {
   constexpr bool GATED = EPI == EPI_GATED;
   // per wave: one tile of 16 rows x 128 k (4 KB) of W and one of x between load and MFMA layout; after
   // the stream the region holds the wave's partial output tiles
@@ -337,15 +332,8 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 #pragma unroll
     for (int j = 0; j < MT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  // The blocks walk K from different starting points and wrap around: rows lie a multiple of kilobytes apart, and
-  // blocks that all read the same columns of their rows at the same time crowd into few memory channels.  The
-  // start depends on the block's place only, so the order of the sum does too.
   const int ngroups = (K + 127) / 128;
-  const int rounds = (ngroups + SK_WAVES * UNR - 1) / (SK_WAVES * UNR);
-  const int first_round = rotate ? (int)(blockIdx.x % (unsigned)rounds) : 0;
-  for (int rnd = 0; rnd < rounds; ++rnd) {
-    const int c0 = (rnd + first_round < rounds ? rnd + first_round : rnd + first_round - rounds) * (SK_WAVES * UNR) + wave * UNR;
-    if (c0 >= ngroups) continue;  // uniform in the wave
+  for (int c0 = wave * UNR; c0 < ngroups; c0 += SK_WAVES * UNR) {
     bf16x8 wreg[UNR][NTB][4], xreg[UNR][MT][4];
 #pragma unroll
     for (int u = 0; u < UNR; ++u) {
@@ -370,14 +358,9 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
       for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-          if (XD) {  // q is the k-step: lane (r, g) takes row r, piece 4 q + g
-            const int m = t * 16 + r, kx = (c0 + u) * 128 + (4 * q + g) * 8;
-            if (t * 16 < M) xreg[u][t][q] = *reinterpret_cast<const bf16x8*>(x + (size_t)(m < M ? m : 0) * ldx + (kx < K ? kx : 0));
-          } else {
-            const int m = t * 16 + 4 * q + lrow;
-            if (t * 16 + 4 * q < M)  // uniform: whole instructions fall away for few rows
-              xreg[u][t][q] = *reinterpret_cast<const bf16x8*>(x + (size_t)(m < M ? m : 0) * ldx + (kok ? k : 0));
-          }
+          const int m = t * 16 + 4 * q + lrow;
+          if (t * 16 + 4 * q < M)  // uniform: whole instructions fall away for few rows
+            xreg[u][t][q] = *reinterpret_cast<const bf16x8*>(x + (size_t)(m < M ? m : 0) * ldx + (kok ? k : 0));
         }
     }
 #pragma unroll
@@ -402,16 +385,6 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
 #pragma unroll
       for (int j = 0; j < MT; ++j) {
         if (j * 16 >= M) break;  // uniform: the tile has no rows, its sums stay zero
-        if (XD) {
-#pragma unroll
-          for (int st = 0; st < 4; ++st) {
-            const bool inside = j * 16 + r < M && (c0 + u) * 128 + (4 * st + g) * 8 < K;
-            const bf16x8 bx = inside ? xreg[u][j][st] : zero;
-#pragma unroll
-            for (int i = 0; i < NTB; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i][st], bx, acc[i][j], 0, 0, 0);
-          }
-          continue;
-        }
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           const int row = 4 * q + lrow;
@@ -542,20 +515,19 @@ __global__ void __launch_bounds__(SK_WAVES* WAVE)
   }
 }
 
-template <int NTB, int MT, int EPI, bool XD = false>
+template <int NTB, int MT, int EPI>
 static void launch_skinny(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                           int out_dtype, long ldo, int M, int N, int K, int tile2_offset, int act, int rows_per_block,
                           hipStream_t stream, RowScale scale, RopeEpilogue rope = RopeEpilogue{},
                           ResidEpilogue res = ResidEpilogue{}) {
   const int blocks = ceil_div(N, rows_per_block);
   const bool fb = bias != nullptr && bias_dtype == FMS_F32;
-  static const int rotate = getenv("FMSAMD_EXP_NOROT") ? 0 : 1;
   constexpr int SK_WAVES = 8;
   constexpr int UNR = (NTB + MT) <= 2 ? 2 : 1;
 #define FMS_SK(O, B)                                                                                 \
-  skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, EPI, O, B, XD><<<blocks, SK_WAVES * WAVE, 0, stream>>>(     \
+  skinny_bf16_kernel<SK_WAVES, UNR, NTB, MT, EPI, O, B><<<blocks, SK_WAVES * WAVE, 0, stream>>>(     \
       (const bf16*)x, ldx, (const bf16*)w, (const B*)bias, (O*)out, ldo, M, N, K, tile2_offset, act, rows_per_block,  \
-      scale, rope, res, rotate)
+      scale, rope, res)
   if (out_dtype == FMS_BF16) {
     if (fb)
       FMS_SK(bf16, float);
@@ -584,14 +556,7 @@ static int skinny_x_rows(int M) { return ceil_div(M, 4) * 4; }
 // gemm_wide.hip, which have to cut so short a K into slices that meet in memory and need a second kernel
 // (measured at K = 4096: 13.5 against 17.2 us for 6144 weight rows, 11.3 against 14.5 for 4096; at K = 14336, and
 // from 33 rows on, where every block reads more of x than of W, the wide kernels win).
-static int exp_xd() {
-  static const int v = getenv("FMSAMD_EXP_XD") ? atoi(getenv("FMSAMD_EXP_XD")) : 0;
-  return v;
-}
-static bool skinny_takes_many_rows(int M, int N, int K) {
-  if (exp_xd() && M > 16 && M <= 64 && K <= exp_xd()) return true;
-  return M > 16 && M <= 32 && K <= 8192;
-}
+static bool skinny_takes_many_rows(int M, int N, int K) { return M > 16 && M <= 32 && K <= 8192; }
 
 static int skinny_rows_per_block(int N, int M) {
   int best = 0;
@@ -639,20 +604,14 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
     return wide_product(EPI_PLAIN, x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, scale, RopeEpilogue{},
                         ResidEpilogue{}, workspace, workspace_bytes, stream);
   const int rows = skinny_rows_per_block(N, M);
-#define FMS_LS(NTB, MT, XD) \
-  launch_skinny<NTB, MT, EPI_PLAIN, XD>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, rows, stream, scale)
-#define FMS_LS_MT(NTB)           \
-  do {                           \
-    if (M <= 16)                 \
-      FMS_LS(NTB, 1, false);     \
-    else if (exp_xd() && M <= 32) \
-      FMS_LS(NTB, 2, true);      \
-    else if (M <= 32)            \
-      FMS_LS(NTB, 2, false);     \
-    else if (M <= 48)            \
-      FMS_LS(NTB, 3, true);      \
-    else                         \
-      FMS_LS(NTB, 4, true);      \
+#define FMS_LS(NTB, MT) \
+  launch_skinny<NTB, MT, EPI_PLAIN>(x, ldx, w, bias, bias_dtype, out, out_dtype, ldo, M, N, K, 0, 0, rows, stream, scale)
+#define FMS_LS_MT(NTB)  \
+  do {                  \
+    if (M <= 16)        \
+      FMS_LS(NTB, 1);   \
+    else                \
+      FMS_LS(NTB, 2);   \
   } while (0)
   if (rows > 16)
     FMS_LS_MT(2);
@@ -721,20 +680,14 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
     return wide_product(EPI_ROPE, x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, scale, rope,
                         ResidEpilogue{}, workspace, workspace_bytes, stream);
   const int rows = skinny_rows_per_block(N, M);
-#define FMS_LR(NTB, MT, XD) \
-  launch_skinny<NTB, MT, EPI_ROPE, XD>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
-#define FMS_LR_MT(NTB)           \
-  do {                           \
-    if (M <= 16)                 \
-      FMS_LR(NTB, 1, false);     \
-    else if (exp_xd() && M <= 32) \
-      FMS_LR(NTB, 2, true);      \
-    else if (M <= 32)            \
-      FMS_LR(NTB, 2, false);     \
-    else if (M <= 48)            \
-      FMS_LR(NTB, 3, true);      \
-    else                         \
-      FMS_LR(NTB, 4, true);      \
+#define FMS_LR(NTB, MT) \
+  launch_skinny<NTB, MT, EPI_ROPE>(x, ldx, w, bias, bias_dtype, out, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, scale, rope)
+#define FMS_LR_MT(NTB)  \
+  do {                  \
+    if (M <= 16)        \
+      FMS_LR(NTB, 1);   \
+    else                \
+      FMS_LR(NTB, 2);   \
   } while (0)
   if (rows > 16)
     FMS_LR_MT(2);
@@ -793,21 +746,15 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
     return wide_product(EPI_RESID, x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, scale,
                         RopeEpilogue{}, res, workspace, workspace_bytes, stream);
   }
-#define FMS_LX(NTB, MT, XD)                                                                                          \
-  launch_skinny<NTB, MT, EPI_RESID, XD>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, \
+#define FMS_LX(NTB, MT)                                                                                              \
+  launch_skinny<NTB, MT, EPI_RESID>(x, ldx, w, bias, bias_dtype, scaled, FMS_BF16, ldo, M, N, K, 0, 0, rows, stream, \
                                     scale, RopeEpilogue{}, res)
-#define FMS_LX_MT(NTB)           \
-  do {                           \
-    if (M <= 16)                 \
-      FMS_LX(NTB, 1, false);     \
-    else if (exp_xd() && M <= 32) \
-      FMS_LX(NTB, 2, true);      \
-    else if (M <= 32)            \
-      FMS_LX(NTB, 2, false);     \
-    else if (M <= 48)            \
-      FMS_LX(NTB, 3, true);      \
-    else                         \
-      FMS_LX(NTB, 4, true);      \
+#define FMS_LX_MT(NTB)  \
+  do {                  \
+    if (M <= 16)        \
+      FMS_LX(NTB, 1);   \
+    else                \
+      FMS_LX(NTB, 2);   \
   } while (0)
   if (rows > 16)
     FMS_LX_MT(2);
