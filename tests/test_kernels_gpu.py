@@ -757,3 +757,13 @@ def test_kernels_refuse_what_they_cannot_do(ops):
         ops.embed(torch.zeros(2, dtype=torch.int32), torch.zeros(4, 4))  # CPU tensors: no CPU path
     with pytest.raises((KernelError, ValueError)):
         ops.sample(dev(torch.zeros(1, 8)), True, 0.0, 0, dev(torch.zeros(1, 2, dtype=torch.int64)))
+
+
+def test_the_probes_measure_this_gpu(ops):
+    """What the benchmark divides by: a kernel that only reads and one that only issues matrix instructions.  On an
+    MI355X the first lies between a quarter of and the whole published 8 TB/s, the second between a fifth of and the
+    whole published 2.5 PFLOP/s; a probe whose loop the compiler removed, or that counts its work wrongly, falls outside."""
+    read, mfma = ops.measured_peaks(read_mib=256, repeats=3)
+    assert 2.0e12 < read < 8.0e12, f"a pure read measured at {read / 1e12:.2f} TB/s"
+    assert 0.5e15 < mfma < 2.5e15, f"matrix instructions measured at {mfma / 1e15:.2f} PFLOP/s"
+

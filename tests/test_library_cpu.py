@@ -916,6 +916,19 @@ def test_sampling_uniforms_are_a_function_of_seed_and_counter():
         SamplingParams(do_sample=True, temperature=0.0)
 
 
+def test_bench_refuses_more_than_one_gpu():
+    """The benchmark's contract: for N > 1 one line that says so, and exit code 2 (this library runs on one GPU)."""
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for args, env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "4"})):
+        run = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *args], capture_output=True, text=True,
+                             env={**os.environ, **env}, timeout=120)
+        assert run.returncode == 2
+        assert len(run.stdout.strip().splitlines()) == 1 and "one GPU" in run.stdout
+
+
 def test_no_gpu_means_a_loud_failure():
     if torch.cuda.is_available():
         pytest.skip("this machine has a GPU")
