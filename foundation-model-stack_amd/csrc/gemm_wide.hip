@@ -74,28 +74,6 @@ __global__ void __launch_bounds__(512)
   const int g_end = g_begin + groups_per_slice < ngroups ? g_begin + groups_per_slice : ngroups;
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  if (MODE != WD_PARTIAL) {  // 1 / rms of the rows of x, if their norm was left to this product
-    constexpr int RPW = MT * 2;
-    if (o.scale.partials != nullptr) {
-      float sum[RPW];
-#pragma unroll
-      for (int k = 0; k < RPW; ++k) sum[k] = 0.f;
-      for (int i = lane; i < o.scale.count; i += WAVE)
-#pragma unroll
-        for (int k = 0; k < RPW; ++k) {
-          const int m = wave * RPW + k < M ? wave * RPW + k : M - 1;
-          sum[k] += o.scale.partials[(size_t)m * o.scale.count + i];
-        }
-#pragma unroll
-      for (int k = 0; k < RPW; ++k) {
-        const float total = wave_sum(sum[k]);
-        if (lane == 0) row_scale[wave * RPW + k] = rsqrtf(total * o.scale.inv_width + o.scale.eps);
-      }
-    } else if (lane < RPW) {
-      row_scale[wave * RPW + lane] = 1.f;
-    }
-  }
-
   // x pieces of a step: MT * 16 rows x 16 pieces, dealt over the 512 threads (row = id / 16, piece = id % 16).
   // Loads never sit behind a branch and their data is not touched before the step that uses it (either makes
   // the compiler wait for every load in flight): a piece out of range is read from a valid address, and is
@@ -155,6 +133,34 @@ __global__ void __launch_bounds__(512)
   for (int d = 0; d < WD_DEPTH - 1; ++d) {
     load_x(group_of(d), xr[d]);
     load_w(group_of(d), wr[d]);
+  }
+  if (MODE != WD_PARTIAL) {
+    // 1 / rms of the rows of x, if their norm was left to this product.  The partial sums are asked for behind the
+    // stream's first loads and all at once: in front of them, one round trip after the other, they kept the
+    // stream from starting for as long as four of its steps take.
+    constexpr int RPW = MT * 2, PRE = 4;  // rows a wave, loads a row that are under way together (256 sums)
+    if (o.scale.partials != nullptr) {
+      float pre[RPW][PRE];
+#pragma unroll
+      for (int k = 0; k < RPW; ++k)
+#pragma unroll
+        for (int j = 0; j < PRE; ++j) {
+          const int m = wave * RPW + k < M ? wave * RPW + k : M - 1, i = lane + j * WAVE;
+          pre[k][j] = o.scale.partials[(size_t)m * o.scale.count + (i < o.scale.count ? i : 0)];
+        }
+#pragma unroll
+      for (int k = 0; k < RPW; ++k) {
+        const int m = wave * RPW + k < M ? wave * RPW + k : M - 1;
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < PRE; ++j) sum += lane + j * WAVE < o.scale.count ? pre[k][j] : 0.f;
+        for (int i = lane + PRE * WAVE; i < o.scale.count; i += WAVE) sum += o.scale.partials[(size_t)m * o.scale.count + i];
+        const float total = wave_sum(sum);
+        if (lane == 0) row_scale[wave * RPW + k] = rsqrtf(total * o.scale.inv_width + o.scale.eps);
+      }
+    } else if (lane < RPW) {
+      row_scale[wave * RPW + lane] = 1.f;
+    }
   }
   for (int t = 0; t < n_steps; t += WD_DEPTH) {
 #pragma unroll
@@ -291,12 +297,49 @@ __global__ void __launch_bounds__(256)
   const int n = blockIdx.x * WAVE + lane;
   if (m >= M) return;  // whole waves
   const bool live = n < N;
+  const int nn = live ? n : 0;  // a lane past the end reads column 0 and stores nothing
 
-  // The slices are added in their order, four loads under way at a time.
-  auto add_slices = [&](const float* p) {
-    const size_t stride = (size_t)M * rows;
+  // Every load that does not wait for another one's result is asked for here, at once and not behind a branch:
+  // the first slices, the partial sums of the rows' norm, the row's position and sequence, the stream and the next
+  // norm's weight.  One after the other they were six to eight round trips to memory for a kernel that moves a
+  // few megabytes.  What is out of range is read from a valid address and set aside where it is used.
+  constexpr int FIRST = 8, PRE = 4;
+  const size_t stride = (size_t)M * rows;
+  const float* const pv = part + (size_t)m * rows + nn;
+  const float* const pu = pv + tile2_offset;
+  float av[FIRST], au[FIRST], pre[PRE];  // au: the up half of a gated product, unused otherwise
+#pragma unroll
+  for (int s = 0; s < FIRST; ++s) {
+    const size_t at = (size_t)(s < slices ? s : 0) * stride;
+    av[s] = pv[at];
+    if (EPI == EPI_GATED) au[s] = pu[at];
+  }
+  if (scale.partials != nullptr) {  // uniform
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) {
+      const int i = lane + j * WAVE;
+      pre[j] = scale.partials[(size_t)m * scale.count + (i < scale.count ? i : 0)];
+    }
+  }
+  int pos = 0, seq = -1;
+  if (EPI == EPI_ROPE) pos = rope.positions[m], seq = rope.seq_of_token[m];
+  float stream_in = 0.f, nw = 1.f, bias_v = 0.f, bias_u = 0.f;
+  if (EPI == EPI_RESID) {
+    stream_in = res.resid[(size_t)m * res.ldr + nn];
+    if (res.norm_w != nullptr) nw = res.norm_w_f32 ? ((const float*)res.norm_w)[nn] : to_f32(((const bf16*)res.norm_w)[nn]);
+  }
+  if (bias) {
+    bias_v = to_f32(bias[nn]);
+    if (EPI == EPI_GATED) bias_u = to_f32(bias[tile2_offset + nn]);
+  }
+
+  // The slices are added in their order, whatever the launch looks like.
+  auto add_slices = [&](const float* p, const float (&first)[FIRST]) {
     float sum = 0.f;
-    int s = 0;
+#pragma unroll
+    for (int s = 0; s < FIRST; ++s)
+      if (s < slices) sum += first[s];
+    int s = FIRST;
     for (; s + 4 <= slices; s += 4) {
       const float a0 = p[(size_t)s * stride], a1 = p[(size_t)(s + 1) * stride], a2 = p[(size_t)(s + 2) * stride],
                   a3 = p[(size_t)(s + 3) * stride];
@@ -305,15 +348,14 @@ __global__ void __launch_bounds__(256)
     for (; s < slices; ++s) sum += p[(size_t)s * stride];
     return sum;
   };
-  float v = 0.f, u = 0.f;
-  if (live) {
-    v = add_slices(part + (size_t)m * rows + n);
-    if (EPI == EPI_GATED) u = add_slices(part + (size_t)m * rows + tile2_offset + n);
-  }
+  float v = add_slices(pv, av), u = 0.f;
+  if (EPI == EPI_GATED) u = add_slices(pu, au);
   float row_scale = 1.f;
   if (scale.partials != nullptr) {
     float sum = 0.f;
-    for (int i = lane; i < scale.count; i += WAVE) sum += scale.partials[(size_t)m * scale.count + i];
+#pragma unroll
+    for (int j = 0; j < PRE; ++j) sum += lane + j * WAVE < scale.count ? pre[j] : 0.f;
+    for (int i = lane + PRE * WAVE; i < scale.count; i += WAVE) sum += scale.partials[(size_t)m * scale.count + i];
     row_scale = rsqrtf(wave_sum(sum) * scale.inv_width + scale.eps);
   }
   v *= row_scale;
@@ -321,18 +363,13 @@ __global__ void __launch_bounds__(256)
 
   if (EPI == EPI_GATED) {
     if (!live) return;
-    if (bias) {
-      v += to_f32(bias[n]);
-      u += to_f32(bias[tile2_offset + n]);
-    }
-    out[(size_t)m * ldo + n] = from_f32<OutT>(sk_activate(v, act) * u);
+    out[(size_t)m * ldo + n] = from_f32<OutT>(sk_activate(v + bias_v, act) * (u + bias_u));
   } else if (EPI == EPI_ROPE) {
-    if (bias && live) v += to_f32(bias[n]);
+    v += bias_v;
     const float partner = __shfl_xor(v, 1, WAVE);  // the other element of the rotary pair (N is even)
     if (!live) return;
     const int D = rope.head_dim;
     const int hh = n / D, d = n - hh * D;
-    const int pos = rope.positions[m], seq = rope.seq_of_token[m];
     if (hh < rope.nheads + rope.kvheads && rope.cos_t != nullptr && d < rope.rot_dim) {
       const int tpos = pos < 0 ? 0 : (pos < rope.max_pos ? pos : rope.max_pos - 1);  // the host has checked the range
       const float c = rope.cos_t[(size_t)tpos * (rope.rot_dim / 2) + d / 2];
@@ -359,12 +396,8 @@ __global__ void __launch_bounds__(256)
   } else if (EPI == EPI_RESID) {
     float stream = 0.f;
     if (live) {
-      if (bias) v += to_f32(bias[n]);
-      stream = res.resid[(size_t)m * res.ldr + n] + v;
+      stream = stream_in + (v + bias_v);
       res.resid[(size_t)m * res.ldr + n] = stream;
-      float nw = 1.f;
-      if (res.norm_w != nullptr)
-        nw = res.norm_w_f32 ? ((const float*)res.norm_w)[n] : to_f32(((const bf16*)res.norm_w)[n]);
       out[(size_t)m * ldo + n] = from_f32<OutT>(stream * nw);
     }
     float sq = stream * stream;  // sums over the groups of 16 neighbouring columns
@@ -373,8 +406,7 @@ __global__ void __launch_bounds__(256)
     if ((lane & 15) == 0 && n / 16 < res.tiles) res.partials[(size_t)m * res.tiles + n / 16] = sq;
   } else {
     if (!live) return;
-    if (bias) v += to_f32(bias[n]);
-    out[(size_t)m * ldo + n] = from_f32<OutT>(v);
+    out[(size_t)m * ldo + n] = from_f32<OutT>(v + bias_v);
   }
 }
 
