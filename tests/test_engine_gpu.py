@@ -772,6 +772,38 @@ def test_command_line(lib, folders):
     assert tok.decode((ids + P.greedy_generate(weights, cfg, ids, 16, stop=tok.eos_token_id))[1:]) in out
 
 
+def test_chat_command(lib, folders):
+    """bin/fms_chat, the reference's scripts/chat.py (:196-243): two questions on piped input.  With --deterministic the
+    answers are the plain implementation's greedy continuations of the conversation in the Llama layout, the second
+    one with the first question and its answer in front."""
+    from fms_amd.tokenizers import CharTokenizer
+
+    name = "A"  # its vocabulary is the character tokenizer's
+    cfg, weights = plain(folders, name)
+    tok = CharTokenizer()
+    bos, eos = tok.bos_token_id, tok.eos_token_id
+
+    def plain_answer(ids):
+        new = P.greedy_generate(weights, cfg, ids, 12, stop=eos)
+        return new[:new.index(eos)] if eos in new else new
+
+    ids = [bos] + tok.encode("<<SYS>>\nshort\n<</SYS>>\n\n") + tok.encode("[INST]one[/INST]")
+    first = plain_answer(ids)
+    ids += first + [eos] + tok.encode("[INST]two[/INST]")
+    second = plain_answer(ids)
+
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "fms_chat"), "--architecture", "hf_pretrained", "--model_path", folders[name],
+           "--tokenizer", "char_tokenizer", "--default_dtype", "fp32", "--max_new_tokens", "12", "--deterministic",
+           "--system_message", "short"]
+    env = dict(os.environ, PYTHONIOENCODING="utf-8")
+    proc = subprocess.run(cmd, input="one\ntwo\n/buffer\n".encode(), stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=110, env=env)
+    assert proc.returncode == 0, proc.stderr.decode(errors="replace")
+    out = proc.stdout.decode("utf-8")
+    assert "loading complete" in out and out.rstrip().endswith("Exiting...")
+    assert tok.decode(first) in out and tok.decode(second) in out
+    assert f"The conversation has {len(ids) + len(second) + 1} tokens:" in out
+
+
 def test_a_type_asked_for_casts_a_checkpoint_stored_in_32_bit(lib, tmp_path):
     """tests/models/test_getmodel_datatype.py:58-73: data_type wins over the checkpoint's type.  The bfloat16
     model made from a float32 folder runs the bfloat16 kernels and follows the plain implementation."""

@@ -905,6 +905,50 @@ def test_command_line_refusals(capsys):
         assert "not a registered variant" in capsys.readouterr().err
 
 
+def test_chat_keeps_the_conversation_in_the_llama_layout(capsys):
+    """scripts/chat.py:162-173 (the layout), :217-243 (a turn), :245-281 (the commands): the conversation is one list of
+    token ids, bos, the system message between its marks, then [INST] question [/INST] answer eos for every turn; the
+    model sees all of it at every question; nothing after an answer's end is kept."""
+    import io
+
+    from fms_amd.cli.chat import Conversation, build_parser, main, run_line
+    from fms_amd.tokenizers import CharTokenizer
+
+    tok = CharTokenizer()
+    seen = []
+
+    def answer(ids, max_new_tokens):
+        seen.append((list(ids), max_new_tokens))
+        reply = tok.encode(f"answer {len(seen)}") + [tok.eos_token_id] + tok.encode("never kept")
+        return reply[:max_new_tokens]
+
+    talk = Conversation(tok, answer, system_message="be brief", max_new_tokens=50)
+    out = io.StringIO()
+    assert run_line(talk, "hello\n", out) and run_line(talk, "   \n", out)  # an empty line asks nothing
+    assert run_line(talk, "/set max_new_tokens=6\n", out) and talk.max_new_tokens == 6
+    assert run_line(talk, "and again\n", out)
+    assert run_line(talk, "/set max_new_tokens\n", out) and run_line(talk, "/nonsense\n", out) and run_line(talk, "/help\n", out)
+    assert run_line(talk, "/buffer\n", out)
+    assert not run_line(talk, "/quit\n", out)
+    bos, eos = [tok.bos_token_id], [tok.eos_token_id]
+    first = bos + tok.encode("<<SYS>>\nbe brief\n<</SYS>>\n\n") + tok.encode("[INST]hello[/INST]")
+    second = first + tok.encode("answer 1") + eos + tok.encode("[INST]and again[/INST]")
+    assert seen == [(first, 50), (second, 6)]
+    assert talk.ids == second + tok.encode("answer") + eos  # six tokens of "answer 2", then the end mark
+    printed = out.getvalue().splitlines()
+    assert printed[0] == "answer 1" and printed[1] == "answer"
+    assert "usage: /set max_new_tokens=100" in printed and "Unknown command: /nonsense" in printed
+    assert f"The conversation has {len(talk.ids)} tokens:" in printed and "Exiting..." == printed[-1]
+    assert Conversation(tok, answer).ids == bos  # no system message, no marks
+
+    options = {a.dest for a in build_parser()._actions}
+    assert {"device_type", "architecture", "variant", "model_path", "model_source", "tokenizer", "no_use_cache", "compile",
+            "compile_mode", "deterministic", "distributed", "max_new_tokens", "system_message"} <= options
+    assert main(["--tokenizer", "char_tokenizer", "--variant", "micro", "--distributed"]) == 2
+    assert main(["--tokenizer", "char_tokenizer"]) == 2
+    capsys.readouterr()
+
+
 def test_sampling_uniforms_are_a_function_of_seed_and_counter():
     from fms_amd.sampling import SamplingParams, request_seed, uniform
 
