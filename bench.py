@@ -38,8 +38,8 @@ def main() -> int:
     ap.add_argument("--prompt-min", type=int, default=128, help="shortest prompt of the decode batches")
     ap.add_argument("--prompt-max", type=int, default=2048, help="longest prompt of the decode batches")
     ap.add_argument("--skip-points", action="store_true", help="leave out the further points (batch 1 and 64, long contexts, the 7B shape)")
-    ap.add_argument("--with-70b", action="store_true",
-                    help="add the Llama-3-70B shape at batch 16, prompts of 256..4096, 128 steps (141 GB of weights: minutes)")
+    ap.add_argument("--skip-70b", action="store_true", help="leave out the point at the Llama-3-70B shape (141 GB of weights)")
+    ap.add_argument("--with-70b", action="store_true", help="accepted for older command lines: the 70B point is measured unless --skip-70b says no")
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="run one phase only (for profiling); the record then lacks the other")
@@ -212,12 +212,17 @@ def main() -> int:
         point("llama2_7b_b8", *decode(8, 256, 8, model=other, prompt_min=64, prompt_max=1024))
         del other
         torch.cuda.empty_cache()
-        if args.with_70b:
-            big = fms_amd.get_model("llama", "3-70b", data_type="bf16", device_type="cuda", random_seed=args.seed,
-                                    max_expected_seq_len=8192)
-            point("llama3_70b_b16", *decode(16, 128, 4, model=big, prompt_min=256, prompt_max=4096))
-            del big
-            torch.cuda.empty_cache()
+        # the Llama-3-70B shape on the one GPU: batch 16, prompts of 256..4096 tokens, 128 decode steps; 141 GB of
+        # weights and 25 GB of cache beside the models above, so only where that much memory is free
+        if not args.skip_70b:
+            if torch.cuda.mem_get_info()[0] > 200e9:
+                big = fms_amd.get_model("llama", "3-70b", data_type="bf16", device_type="cuda", random_seed=args.seed,
+                                        max_expected_seq_len=8192)
+                point("llama3_70b_b16", *decode(16, 128, 4, model=big, prompt_min=256, prompt_max=4096))
+                del big
+                torch.cuda.empty_cache()
+            else:
+                points["llama3_70b_b16"] = None  # not measured: less than 200 GB free on this GPU
 
     record = {
         "metric": f"decode tok/s at batch {args.batch} (llama {args.variant} shape, {args.context} context); prefill tok/s at {args.prefill_tokens} tokens",
