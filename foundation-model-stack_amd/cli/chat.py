@@ -9,7 +9,8 @@ describes (:162-173):
 
     <bos> <<SYS>>\\n system \\n<</SYS>>\\n\\n [INST] question [/INST] answer <eos> [INST] question [/INST] answer <eos> ...
 
-and every question runs the whole list through `generate` again, as the reference does (:224-240).  Lines that
+The reference runs the whole list through `generate` at every question (:224-240); here the conversation
+keeps its sequence in the cache, and a question runs only the tokens that are new.  Lines that
 start with a slash are commands (/help, /set max_new_tokens=N, /buffer, /quit); anything else goes to the model.
 (The reference's code closes the system message with a second "<<SYS>>", :184; the layout it cites closes it
 with "<</SYS>>", which is what is written here.)
@@ -50,8 +51,9 @@ class Conversation:
 
     def ask(self, text: str) -> str:
         eos = self.tokenizer.eos_token_id
-        self.ids += list(self.tokenizer.encode(B_INST + text + E_INST))
-        new = [int(t) for t in self.answer(list(self.ids), self.max_new_tokens)]
+        asked = list(self.tokenizer.encode(B_INST + text + E_INST))
+        new = [int(t) for t in self.answer(self.ids + asked, self.max_new_tokens)]  # a question that is refused is not kept
+        self.ids += asked
         if eos in new:  # nothing after the end of the answer is kept
             new = new[:new.index(eos)]
         self.ids += new + [eos]
@@ -124,10 +126,9 @@ def main(argv=None, stdin=None, stdout=None) -> int:
         print("--variant is needed with --architecture", args.architecture, file=sys.stderr)
         return 2
 
-    import torch
-
     from .. import get_model
-    from ..generation import generate
+    from ..engine import Engine
+    from ..sampling import SamplingParams, choose
     from ..tokenizers import get_tokenizer
 
     print("loading model", file=stdout, flush=True)
@@ -144,18 +145,25 @@ def main(argv=None, stdin=None, stdout=None) -> int:
     tokenizer = get_tokenizer(args.tokenizer)
     print("loading complete", file=stdout, flush=True)
 
+    # The conversation keeps its place in the cache: a question runs only the tokens that are new since the last
+    # answer (the reference's script runs the whole conversation again at every question, scripts/chat.py:224-240).
+    engine = Engine(model, max_tokens=model.spec.max_seq_len, max_slots=1)
+    slot = engine.new_sequence()
+    sampling = SamplingParams(do_sample=not args.deterministic, temperature=args.temperature, top_k=args.top_k)
     turn = [0]
 
     def answer(ids: List[int], max_new_tokens: int) -> List[int]:
+        held = engine.length(slot)  # the conversation up to the last token that was fed
         room = model.spec.max_seq_len - len(ids)
         if room < 1:
             raise ValueError(f"the conversation has {len(ids)} tokens, the model takes {model.spec.max_seq_len}")
         turn[0] += 1
-        result = generate(model, torch.tensor(ids, dtype=torch.long), max_new_tokens=min(max_new_tokens, room),
-                          max_seq_len=model.spec.max_seq_len, use_cache=True, do_sample=not args.deterministic,
-                          temperature=args.temperature, top_k=args.top_k, eos_token_id=tokenizer.eos_token_id,
-                          seed=42 if args.deterministic else turn[0])
-        return result[len(ids):].tolist()
+        seed = 42 if args.deterministic else turn[0]
+        logits = engine.step([slot], [ids[held:]], "last")
+        new = choose(logits, sampling, [seed], [0]).tolist()
+        while new[-1] != tokenizer.eos_token_id and len(new) < min(max_new_tokens, room):
+            new += engine.decode_and_choose([slot], [new[-1]], sampling, [seed], [len(new)])
+        return new
 
     conversation = Conversation(tokenizer, answer, args.system_message, args.max_new_tokens)
     print('Enter your prompts/questions or "/help" for usage instructions.\n', file=stdout, flush=True)
