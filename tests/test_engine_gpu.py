@@ -148,6 +148,50 @@ def test_first_tokens_and_chunks(lib, folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "E"])
+def test_steps_of_any_mix(lib, folders, name, dtype):
+    """More than the loop above it asks of the step function: in one step some sequences bring a piece of their prompt,
+    others one token, and new ones join while the rest go on; sequences end at different times and their slots are
+    taken again.  A seeded random schedule; every logit is compared with the plain implementation's for the whole
+    sequence."""
+    import random
+
+    from fms_amd.engine import Engine
+
+    cfg, weights = plain(folders, name)
+    engine = Engine(get(lib, folders, name, dtype), max_tokens=6 * 192, max_slots=4)
+    rng = random.Random(17)
+    waiting = [tokens_for(name, rng.choice((3, 40, 64, 65, 130, 180)), 300 + i) for i in range(9)]
+    running = []  # [ids, slot, tokens fed so far, logits]
+    finished = []
+    n_mixed = 0
+    while waiting or running:
+        while waiting and len(running) < 4 and (not running or rng.random() < 0.5):
+            running.append([waiting.pop(), engine.new_sequence(), 0, []])
+        pieces = []
+        for seq in running:
+            left = len(seq[0]) - seq[2]
+            n = min(left, rng.choice((1, 1, 1, 2, 17, 63, 64, 70)))
+            pieces.append(seq[0][seq[2] : seq[2] + n])
+        n_mixed += len({len(p) == 1 for p in pieces}) == 2
+        logits = engine.step([seq[1] for seq in running], pieces, "all")
+        row = 0
+        for seq, piece in zip(running, pieces):
+            seq[3].append(logits[row : row + len(piece)])
+            seq[2] += len(piece)
+            row += len(piece)
+        assert row == logits.shape[0]
+        for seq in [seq for seq in running if seq[2] == len(seq[0])]:
+            engine.end_sequence(seq[1])
+            running.remove(seq)
+            finished.append(seq)
+        engine.cache.check()
+    assert engine.cache.live_slots() == [] and len(finished) == 9 and n_mixed >= 5
+    for ids, _, _, got in finished:
+        check(torch.cat(got), expect(weights, cfg, ids, dtype), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", sorted(CONFIGS))
 def test_ragged_batches_with_reused_slots(lib, folders, name, dtype):
     """Batches of unequal prompts that go on token by token; shorter requests end earlier;

@@ -124,6 +124,43 @@ def test_ragged_batches_with_early_ends_and_reused_slots(shape, dtype):
             check(torch.cat(s["got"]), expect(shape.weights, shape.cfg, s["ids"], dtype), dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_steps_of_any_mix(shape, dtype):
+    """In one step some sequences bring a piece of their prompt, others one token, and new ones join while the rest go
+    on (a seeded random schedule): at these sizes a step with any longer piece runs the prefill kernels for all of its
+    rows, a step of single tokens the decode kernels."""
+    import random
+
+    from fms_amd.engine import Engine
+
+    engine = Engine(shape.model(dtype), max_tokens=4 * 448, max_slots=4)
+    rng = random.Random(23)
+    waiting = [shape.tokens(rng.choice((3, 64, 65, 130, 300, 420)), 500 + i) for i in range(7)]
+    running, finished, n_mixed = [], [], 0
+    while waiting or running:
+        while waiting and len(running) < 4 and (not running or rng.random() < 0.5):
+            running.append(dict(ids=waiting.pop(), slot=engine.new_sequence(), at=0, got=[]))
+        pieces = []
+        for seq in running:
+            n = min(len(seq["ids"]) - seq["at"], rng.choice((1, 1, 1, 2, 17, 64, 130)))
+            pieces.append(seq["ids"][seq["at"] : seq["at"] + n])
+        n_mixed += len({len(p) == 1 for p in pieces}) == 2
+        logits = engine.step([seq["slot"] for seq in running], pieces, "all")
+        row = 0
+        for seq, piece in zip(running, pieces):
+            seq["got"].append(logits[row : row + len(piece)])
+            seq["at"] += len(piece)
+            row += len(piece)
+        for seq in [seq for seq in running if seq["at"] == len(seq["ids"])]:
+            engine.end_sequence(seq["slot"])
+            running.remove(seq)
+            finished.append(seq)
+        engine.cache.check()
+    assert engine.cache.live_slots() == [] and len(finished) == 7 and n_mixed >= 4
+    for seq in finished:
+        check(torch.cat(seq["got"]), expect(shape.weights, shape.cfg, seq["ids"], dtype), dtype)
+
+
 def prompt_lengths(n):
     special = [63, 64, 65, 1, 127, 128, 191, 320]
     return [(special[i] if i < len(special) else 2 + (53 * i * i + 17 * i) % 250) for i in range(n)]
