@@ -7,7 +7,9 @@ the library's own generation path (step function, cache, kernels, sampler).  One
 printed: decode tokens/s at batch 8 (`value`), the prefill of 2,048 tokens, the decode step's
 memory roofline (against the published peak and against what a pure read reaches on this GPU now),
 the share of the step's time by kernel class, and further points: decode at batch 1 and 64, at
-batch 8 with every context near 8000 tokens, and the Llama-2-7B shape at batch 8 (256 steps).
+batch 8 with every context near 8000 tokens, the Llama-2-7B shape at batch 8 (256 steps) and the
+Llama-3-70B shape at batch 16 (128 steps).  Decode steps run as generation runs them: the host looks
+at the chosen tokens every `steps_ahead` steps (`--steps-ahead 1`: after every step).
 """
 
 import argparse
@@ -41,6 +43,8 @@ def main() -> int:
     ap.add_argument("--skip-70b", action="store_true", help="leave out the point at the Llama-3-70B shape (141 GB of weights)")
     ap.add_argument("--with-70b", action="store_true", help="accepted for older command lines: the 70B point is measured unless --skip-70b says no")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--steps-ahead", type=int, default=None,
+                    help="decode steps that run before the host looks at their tokens (default: the generation loop's STEPS_AHEAD)")
     ap.add_argument("--only", choices=["decode", "prefill"], default=None,
                     help="run one phase only (for profiling); the record then lacks the other")
     # the workload options of the reference's scripts/benchmark_inference.py:70-87, by their names
@@ -65,6 +69,12 @@ def main() -> int:
     from fms_amd.engine import Engine
     from fms_amd.kernels import ops
     from fms_amd.sampling import SamplingParams, choose
+
+    from fms_amd.generation.loop import STEPS_AHEAD
+
+    if args.steps_ahead is None:
+        args.steps_ahead = STEPS_AHEAD
+    args.steps_ahead = max(1, args.steps_ahead)
 
     # what this GPU delivers now: a kernel that only reads, a kernel that only issues matrix instructions
     read_bps, mfma_flops = ops.measured_peaks()
@@ -106,12 +116,18 @@ def main() -> int:
             logits = engine.step([slots[b] for b in group], prompts, "last")
             first = choose(logits, greedy).tolist()
             tokens = first if tokens is None else tokens + first
-        for _ in range(warmup):
-            tokens = engine.decode_and_choose(slots, tokens, greedy)
+        def run(n):  # n decode steps as the generation loop runs them: the host looks at the tokens every few steps
+            nonlocal tokens
+            done = 0
+            while done < n:
+                ahead = min(args.steps_ahead, n - done)
+                tokens = engine.decode_and_choose_many(slots, tokens, greedy, steps=ahead)[-1]
+                done += ahead
+
+        run(warmup)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(steps):
-            tokens = engine.decode_and_choose(slots, tokens, greedy)
+        run(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         mean_ctx = sum(lens) + batch * (1 + warmup + steps / 2)
@@ -256,6 +272,7 @@ def main() -> int:
             "prompt_len_max": args.prompt_max,
             "prefill_tokens": args.prefill_tokens,
             "cache_page_tokens": 64,
+            "steps_ahead": args.steps_ahead,
         },
         "prefill": {"value": round(pre_tps, 1), "tokens": args.prefill_tokens, "ms": round(pre_ms, 3), "frac": round(pre_frac, 4),
                     "frac_measured": round(pre_frac_measured, 4), "peak_measured_tflops": round(mfma_flops / 1e12, 1)},

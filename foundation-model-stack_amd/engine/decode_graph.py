@@ -75,6 +75,7 @@ class DecodeGraph:
         self.stamps: List[int] = []  # the cache's stamp of every sequence after the last replay
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
+        self.chosen = torch.empty(8, rows, dtype=torch.int32, device=dev)  # [steps, rows]: the tokens of replays that are waited for together
 
     def _run(self) -> None:
         logits = self.engine.model.forward(self.batch, self.engine.cache)
@@ -142,8 +143,19 @@ class DecodeGraph:
                     table[row].copy_(cache.block_table(g, [slot], n_columns=self.table_width)[0], non_blocking=True)
                 self.n_pages[row] = n
 
-    def replay(self) -> List[int]:
-        self.graph.replay()
-        out = self.tokens[: len(self.slots)].tolist()
-        self.next_tokens = out
+    def replay(self, steps: int = 1) -> List[List[int]]:
+        """`steps` replays back to back (every one reads the tokens and positions that the one before left on the
+        device; the block tables already hold the pages of all of them) and one wait for the tokens of all."""
+        n = len(self.slots)
+        if steps == 1:
+            self.graph.replay()
+            out = [self.tokens[:n].tolist()]
+        else:
+            if self.chosen.shape[0] < steps:
+                self.chosen = torch.empty(steps, self.rows, dtype=torch.int32, device=self.tokens.device)
+            for i in range(steps):
+                self.graph.replay()
+                self.chosen[i].copy_(self.tokens)
+            out = self.chosen[:steps, :n].tolist()
+        self.next_tokens = out[-1]
         return out

@@ -89,11 +89,36 @@ class Engine:
     ) -> List[int]:
         """One decode step and the choice of the next token for every sequence: `tokens[b]` is appended to
         `slots[b]`, the chosen tokens come back as host integers.  Replays a captured graph when it can."""
+        return self.decode_and_choose_many(slots, tokens, sampling, seeds, counters, steps=1)[0]
+
+    def decode_and_choose_many(
+        self,
+        slots: Sequence[int],
+        tokens: Sequence[int],
+        sampling: SamplingParams,
+        seeds: Optional[Sequence[int]] = None,
+        counters: Optional[Sequence[int]] = None,
+        steps: int = 1,
+    ) -> List[List[int]]:
+        """`steps` decode steps of the same sequences, each fed what the step before chose: the chosen tokens of
+        every step, `steps` lists of one token per sequence.  With graphs the steps are replayed back to back and
+        the host waits once, for all their tokens; every step is the step that `decode_and_choose` runs, and
+        chooses the same tokens.  All sequences go on for all steps: a caller that watches for stop tokens takes
+        what it wants of the result and ends the sequence (whose cache then holds tokens past its end, which is
+        harmless, as the slot is given back whole).  Room for all steps is made first, or for none of them."""
         slots = [int(s) for s in slots]
         tokens = [int(t) for t in tokens]
+        steps = int(steps)
+        if steps < 1:
+            raise ValueError("at least one step")
         if not self.use_graphs:
-            logits = self.step(slots, [[t] for t in tokens], "last")
-            return choose(logits, sampling, seeds, counters).tolist()
+            out = []
+            for i in range(steps):
+                logits = self.step(slots, [[t] for t in tokens], "last")
+                step_counters = None if counters is None else [c + i for c in counters]
+                tokens = choose(logits, sampling, seeds, step_counters).tolist()
+                out.append(tokens)
+            return out
         if len(set(slots)) != len(slots) or len(tokens) != len(slots):
             raise ValueError("one token per sequence, each sequence once")
         live = set(self.cache.live_slots())
@@ -106,9 +131,9 @@ class Engine:
         # what the sequences looked like before this step: a graph's buffers still describe them only if
         # nothing but the graph's own last replay has touched them since
         before = [self.cache.stamp(s) for s in slots]
-        positions = self.cache.extend_many(slots, [1] * len(slots))  # room for all, or for none
+        positions = self.cache.extend_many(slots, [steps] * len(slots))  # room for all, or for none
         rows = row_bucket(len(slots))
-        longest = max(positions) + 1
+        longest = max(positions) + steps
         how = (sampling.do_sample, float(sampling.temperature), int(sampling.top_k or 0))
         fitting = [k for k in self._graphs if k[0] == rows and k[2:] == how and k[1] >= longest]
         if fitting:
@@ -126,7 +151,7 @@ class Engine:
             graph.load(slots, tokens, positions, seeds or [0] * len(slots), counters or [0] * len(slots))
         graph.stamps = [self.cache.stamp(s) for s in slots]
         self.last_graph = graph
-        return graph.replay()
+        return graph.replay(steps)
 
     def prepare(self, slots, tokens, want) -> StepBatch:
         slots = [int(s) for s in slots]

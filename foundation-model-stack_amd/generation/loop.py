@@ -20,6 +20,11 @@ import torch
 from ..cache import PAGE_TOKENS, pages_for
 from ..sampling import SamplingParams, choose, request_seed
 
+# Decode steps that the loop runs before it looks at their tokens, when nobody asked to see every step: the host
+# then waits once for several steps (its share of a step is a per cent or two), and a request that meets a stop
+# token runs at most this many steps less one for nothing.
+STEPS_AHEAD = 4
+
 
 def plan_batches(
     prompt_lens: Sequence[int],
@@ -94,6 +99,7 @@ def generate_requests(
         return choose(logits, sampling, seeds, counters).tolist()
 
     fused = chooser is None and after_choice is None and hasattr(engine, "decode_and_choose")
+    watched = before_step is not None or on_step is not None or step_times is not None  # someone looks at every step
     for batch in plan_batches([len(p) for p in prompts], max_new_tokens, cache.max_tokens, max_batch, cache.max_seq_len):
         slots = {r: engine.new_sequence() for r in batch}
         alive = list(batch)
@@ -110,7 +116,36 @@ def generate_requests(
                             feed[r] = [int(x) for x in g]
                 t0 = time.time()
                 if fused and step_no > 0 and all(len(feed[r]) == 1 for r in alive):
-                    # decode: the step and the choice in one call (a captured graph when the engine has one)
+                    # decode: the step and the choice in one call (a captured graph when the engine has one).  With
+                    # nobody watching the single steps, several are run before the host looks at their tokens: a
+                    # request that meets a stop token among them ends there, and what it chose after is dropped.
+                    ahead = 1
+                    if watched is False and hasattr(engine, "decode_and_choose_many"):
+                        ahead = min(STEPS_AHEAD, min(min(max_new_tokens - len(results[r]),
+                                                         cache.max_seq_len + 1 - len(prompts[r]) - len(results[r])) for r in alive))
+                    if ahead > 1:
+                        many = engine.decode_and_choose_many(
+                            [slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
+                            [request_seed(seed, r) for r in alive], [len(results[r]) for r in alive], steps=ahead)
+                        still = list(alive)
+                        for tokens in many:
+                            for r, tok in zip(alive, tokens):
+                                if r in still:
+                                    results[r].append(tok)
+                                    if tok in stops:
+                                        still.remove(r)
+                            step_no += 1
+                        last = dict(zip(alive, many[-1]))
+                        for r in alive:
+                            length = len(prompts[r]) + len(results[r])
+                            if r not in still or len(results[r]) >= max_new_tokens or length > cache.max_seq_len:
+                                engine.end_sequence(slots.pop(r))
+                                if r in still:
+                                    still.remove(r)
+                            else:
+                                feed[r] = [last[r]]
+                        alive = still
+                        continue
                     tokens = engine.decode_and_choose(
                         [slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
                         [request_seed(seed, r) for r in alive], [len(results[r]) for r in alive])

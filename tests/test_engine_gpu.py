@@ -643,11 +643,15 @@ def test_replayed_and_eager_steps_choose_the_same_tokens(lib, folders, name, dty
         for sampling in (SamplingParams(do_sample=False), SamplingParams(do_sample=True, temperature=0.9, top_k=20)):
             got[(graphs, sampling.do_sample)] = generate_requests(engine, prompts, max_new_tokens=90, sampling=sampling, seed=5,
                                                                   stop_token_ids=stops)
+            if graphs:
+                # with someone watching every step the loop does not run steps ahead of the host: the same tokens
+                got[("one by one", sampling.do_sample)] = generate_requests(
+                    engine, prompts, max_new_tokens=90, sampling=sampling, seed=5, stop_token_ids=stops, on_step=lambda *a: None)
         engine.cache.check()
         if graphs:
             assert len(set(engine.graph_captures)) >= 3  # the batch went through several row buckets
     for sampled in (False, True):
-        assert got[(True, sampled)] == got[(False, sampled)]
+        assert got[(True, sampled)] == got[(False, sampled)] == got[("one by one", sampled)]
         assert len(set(len(g) for g in got[(True, sampled)])) > 3  # they ended at different times
 
 

@@ -761,6 +761,57 @@ def test_loop_runs_as_many_batches_as_the_requests_need():
     assert engine.cache.live_slots() == []
 
 
+def test_loop_runs_steps_ahead_when_nobody_watches_them(monkeypatch):
+    """With an engine that runs several decode steps in one call (decode_and_choose_many), and no hook, chooser or timer
+    that looks at single steps, the loop asks for up to STEPS_AHEAD steps at a time: never past max_new_tokens or the
+    model's last position, and a request that meets a stop token among them ends there.  The results are those of the
+    loop that goes step by step."""
+    from fms_amd.generation import loop
+    from fms_amd.generation.loop import STEPS_AHEAD
+    from fms_amd.sampling import SamplingParams
+
+    # the prompts' step chooses with the sampling kernel, which needs the GPU: here the largest logit stands in for it
+    monkeypatch.setattr(loop, "choose", lambda logits, sampling, seeds, counters: logits.argmax(-1))
+
+    class Ahead(FakeEngine):
+        def __init__(self, **kw):
+            super().__init__(**kw)
+            self.asked = []
+
+        def decode_and_choose(self, slots, tokens, sampling, seeds=None, counters=None):
+            return self.decode_and_choose_many(slots, tokens, sampling, seeds, counters, steps=1)[0]
+
+        def decode_and_choose_many(self, slots, tokens, sampling, seeds=None, counters=None, steps=1):
+            self.asked.append((len(slots), steps))
+            self.cache.extend_many(slots, [steps] * len(slots))
+            out, tokens = [], list(tokens)
+            for _ in range(steps):
+                tokens = [(t + 1) % self.vocab for t in tokens]
+                out.append(tokens)
+            return out
+
+    greedy = SamplingParams(do_sample=False)
+    prompts = [[10, 11, 12], [50], [20, 21], [97, 98]]
+    step_by_step = generate_requests(FakeEngine(), prompts, max_new_tokens=11, stop_token_ids=[23, 57], chooser=argmax_chooser)
+    engine = Ahead()
+    out = generate_requests(engine, prompts, max_new_tokens=11, stop_token_ids=[23, 57], sampling=greedy)
+    assert out == step_by_step == [list(range(13, 24)), list(range(51, 58)), [22, 23], list(range(99, 110))]
+    # the prompts' step chooses the first token; 10 are left: 4 and 4 ahead, then the 2 that remain.  Request 2 met its
+    # stop token in the first call and request 1 in the second: each ended there, and what it chose after was dropped
+    assert STEPS_AHEAD == 4 and engine.asked == [(4, 4), (3, 4), (2, 2)]
+    assert engine.cache.live_slots() == []
+    # the model's last position bounds the steps ahead: a prompt of 2 in a model of 12 positions takes 11 new tokens,
+    # the last of which is never fed
+    engine = Ahead(max_seq_len=12)
+    assert generate_requests(engine, [[1, 2]], max_new_tokens=500, sampling=greedy) == [list(range(3, 14))]
+    assert engine.asked == [(1, 4), (1, 4), (1, 2)] and engine.cache.live_slots() == []
+    # someone who watches every step gets single steps
+    engine = Ahead()
+    seen = []
+    generate_requests(engine, [[1]], max_new_tokens=6, sampling=greedy, on_step=lambda step, alive, tokens: seen.append(step))
+    assert engine.asked == [(1, 1)] * 5 and seen == list(range(6))
+
+
 def test_padding_helpers_follow_the_reference():
     """tests/utils/test_generate.py:148-198: exact tensors of pad_input_ids."""
     ids, extra = pad_input_ids([torch.arange(1, 5), torch.arange(1, 8)])
