@@ -117,38 +117,19 @@ def generate_requests(
                 t0 = time.time()
                 if fused and step_no > 0 and all(len(feed[r]) == 1 for r in alive):
                     # decode: the step and the choice in one call (a captured graph when the engine has one).  With
-                    # nobody watching the single steps, several are run before the host looks at their tokens: a
-                    # request that meets a stop token among them ends there, and what it chose after is dropped.
+                    # nobody watching the single steps, several are run before the host looks at their tokens, never
+                    # past a request's limit or the model's last position; a request that meets a stop token among
+                    # them ends there, and what it chose after is dropped.
                     ahead = 1
-                    if watched is False and hasattr(engine, "decode_and_choose_many"):
-                        ahead = min(STEPS_AHEAD, min(min(max_new_tokens - len(results[r]),
-                                                         cache.max_seq_len + 1 - len(prompts[r]) - len(results[r])) for r in alive))
+                    if not watched and hasattr(engine, "decode_and_choose_many"):
+                        ahead = min(STEPS_AHEAD, *(min(max_new_tokens - len(results[r]),
+                                                       cache.max_seq_len + 1 - len(prompts[r]) - len(results[r])) for r in alive))
+                    step_args = ([slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
+                                 [request_seed(seed, r) for r in alive], [len(results[r]) for r in alive])
                     if ahead > 1:
-                        many = engine.decode_and_choose_many(
-                            [slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
-                            [request_seed(seed, r) for r in alive], [len(results[r]) for r in alive], steps=ahead)
-                        still = list(alive)
-                        for tokens in many:
-                            for r, tok in zip(alive, tokens):
-                                if r in still:
-                                    results[r].append(tok)
-                                    if tok in stops:
-                                        still.remove(r)
-                            step_no += 1
-                        last = dict(zip(alive, many[-1]))
-                        for r in alive:
-                            length = len(prompts[r]) + len(results[r])
-                            if r not in still or len(results[r]) >= max_new_tokens or length > cache.max_seq_len:
-                                engine.end_sequence(slots.pop(r))
-                                if r in still:
-                                    still.remove(r)
-                            else:
-                                feed[r] = [last[r]]
-                        alive = still
-                        continue
-                    tokens = engine.decode_and_choose(
-                        [slots[r] for r in alive], [feed[r][0] for r in alive], sampling,
-                        [request_seed(seed, r) for r in alive], [len(results[r]) for r in alive])
+                        chosen = engine.decode_and_choose_many(*step_args, steps=ahead)
+                    else:
+                        chosen = [engine.decode_and_choose(*step_args)]
                 else:
                     logits = engine.step([slots[r] for r in alive], [feed[r] for r in alive], "last")
                     tokens = pick(logits, alive, [len(results[r]) for r in alive])
@@ -158,23 +139,28 @@ def generate_requests(
                             if len(given) != len(alive):
                                 raise ValueError("after_choice must return one token per live request")
                             tokens = [int(t) for t in given]
+                    chosen = [tokens]
                 if step_times is not None:
                     step_times.append(time.time() - t0)
                 if on_step is not None:
-                    on_step(step_no, list(alive), list(tokens))
-                still = []
-                for r, tok in zip(alive, tokens):
-                    results[r].append(tok)
-                    length = len(prompts[r]) + len(results[r])
-                    # the token just chosen is not in the cache yet: it may be fed only if a position is left for it
-                    done = tok in stops or len(results[r]) >= max_new_tokens or length > cache.max_seq_len
-                    if done:
+                    on_step(step_no, list(alive), list(chosen[0]))
+                going = list(alive)
+                for tokens in chosen:
+                    for r, tok in zip(alive, tokens):
+                        if r not in going:
+                            continue
+                        results[r].append(tok)
+                        length = len(prompts[r]) + len(results[r])
+                        # the token just chosen is not in the cache yet: it may be fed only if a position is left for it
+                        if tok in stops or len(results[r]) >= max_new_tokens or length > cache.max_seq_len:
+                            going.remove(r)
+                        else:
+                            feed[r] = [tok]
+                    step_no += 1
+                for r in alive:
+                    if r not in going:
                         engine.end_sequence(slots.pop(r))
-                    else:
-                        feed[r] = [tok]
-                        still.append(r)
-                alive = still
-                step_no += 1
+                alive = going
         finally:
             for slot in slots.values():
                 engine.end_sequence(slot)
