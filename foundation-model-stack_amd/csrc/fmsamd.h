@@ -109,7 +109,7 @@ typedef struct {
   float eps;
 } fmsamd_row_scale;
 
-// At most 128 rows: the weights stream once through MFMA registers.  From 17 rows on the product needs a
+// At most 192 rows: the weights stream once through MFMA registers.  From 17 rows on the product needs a
 // workspace of fmsamd_gemm_skinny_workspace(M, rows of W, K) bytes (slices of K meet there).
 long fmsamd_gemm_skinny_workspace(int M, int rows, int K);
 int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
@@ -121,7 +121,7 @@ int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const 
                                   hipStream_t stream);
 // resid += x W^T (+ bias) in float32; scaled = resid * norm_w in bfloat16; partials[M, partial_count] = sums
 // of squares of resid by groups of columns (partial_count as fmsamd_gemm_skinny_residual_partials(M, N, K) says;
-// every entry is written).  At most 128 rows.
+// every entry is written).  At most 192 rows.
 int fmsamd_gemm_skinny_residual_partials(int M, int N, int K);
 int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                      float* resid, long ldr, const void* norm_w, int norm_w_dtype, void* scaled,
@@ -129,7 +129,7 @@ int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const void* w, con
                                      const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
                                      hipStream_t stream);
 
-// qkv = x W^T (+ bias) for at most 128 rows with the rotation and the cache write fused into the epilogue;
+// qkv = x W^T (+ bias) for at most 192 rows with the rotation and the cache write fused into the epilogue;
 // only the query columns of `out` are written
 int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype, void* out,
                                 long ldo, int M, int K, const int* positions, const int* seq_of_token,

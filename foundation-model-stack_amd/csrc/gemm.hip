@@ -10,7 +10,7 @@
 //     long contiguous runs and change to the MFMA layout in LDS, partial
 //     sums meet in LDS.  Epilogues: plain, act(x Wg^T) * (x Wu^T), rotation
 //     and cache write, addition into the residual stream.  The entry points
-//     hand 17 to 128 rows to the kernels of gemm_wide.hip.
+//     hand 17 to 192 rows to the kernels of gemm_wide.hip.
 #include "common.h"
 #include "fmsamd.h"
 #include "gemm_epilogue.h"
@@ -214,7 +214,7 @@ extern "C" int fmsamd_gemm_bf16(const void* a, long lda, const void* w, const vo
 }
 
 // ==========================================================================
-// bfloat16, M <= 16 (and the entry points for M <= 128)
+// bfloat16, M <= 16 (and the entry points for M <= 192)
 // ==========================================================================
 
 // NTB: 16-row tiles of W per block (the second tile starts `tile2_offset` rows after the first).
@@ -588,7 +588,7 @@ static int row_scale_of(const fmsamd_row_scale* in, int K, RowScale* out) {
   return 0;
 }
 
-// out[M, N] = x[M, K] w[N, K]^T (+ bias).  M <= 128.
+// out[M, N] = x[M, K] w[N, K]^T (+ bias).  M <= 192.
 extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                        void* out, int out_dtype, long ldo, int M, int N, int K,
                                        const fmsamd_row_scale* row_scale, void* workspace, long workspace_bytes,
@@ -596,7 +596,7 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   if (M == 0 || N == 0) return 0;
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
-  FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && N > 0 && K > 0, "gemm_skinny_bf16: bad sizes M=%d N=%d K=%d (M <= 128)", M, N, K);
+  FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && N > 0 && K > 0, "gemm_skinny_bf16: bad sizes M=%d N=%d K=%d (M <= 192)", M, N, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N, "gemm_skinny_bf16: leading dimensions too small");
   FMS_REQUIRE(out_dtype == FMS_BF16 || out_dtype == FMS_F32, "gemm_skinny_bf16: unknown output dtype %d", out_dtype);
@@ -623,7 +623,7 @@ extern "C" int fmsamd_gemm_skinny_bf16(const void* x, long ldx, const void* w, c
   return 0;
 }
 
-// out[M, hidden] = act(x Wg^T + bg) * (x Wu^T + bu) with w = [Wg; Wu] stacked, [2*hidden, K].  M <= 128.
+// out[M, hidden] = act(x Wg^T + bg) * (x Wu^T + bu) with w = [Wg; Wu] stacked, [2*hidden, K].  M <= 192.
 extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void* w, const void* bias,
                                              int bias_dtype, void* out, int out_dtype, long ldo, int M, int hidden,
                                              int K, int act, const fmsamd_row_scale* row_scale, void* workspace,
@@ -631,7 +631,7 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
   if (M == 0 || hidden == 0) return 0;
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
-  FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && hidden > 0 && K > 0, "gemm_skinny_gated_bf16: bad sizes M=%d hidden=%d K=%d (M <= 128)",
+  FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && hidden > 0 && K > 0, "gemm_skinny_gated_bf16: bad sizes M=%d hidden=%d K=%d (M <= 192)",
               M, hidden, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_gated_bf16: K=%d and the row stride %ld must be multiples of 8", K,
               ldx);
@@ -652,7 +652,7 @@ extern "C" int fmsamd_gemm_skinny_gated_bf16(const void* x, long ldx, const void
 
 // qkv[M, (H+2K)*D] = x W^T (+ bias) with the rotation of q and k and the cache write of k and v fused into
 // the epilogue: the decode-time twin of fmsamd_gemm_skinny_bf16 followed by fmsamd_rope_kv_write.  Only the
-// query columns of `out` are written.  M <= 128.
+// query columns of `out` are written.  M <= 192.
 extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* w, const void* bias, int bias_dtype,
                                            void* out, long ldo, int M, int K, const int* positions,
                                            const int* seq_of_token, const int* block_table, int table_stride,
@@ -665,7 +665,7 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
   RowScale scale;
   if (row_scale_of(row_scale, K, &scale)) return -1;
   FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && K > 0 && nheads > 0 && kvheads > 0 && head_dim > 0,
-              "qkv_rope_skinny_bf16: bad sizes M=%d K=%d (M <= 128)", M, K);
+              "qkv_rope_skinny_bf16: bad sizes M=%d K=%d (M <= 192)", M, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "qkv_rope_skinny_bf16: K=%d and the row stride %ld must be multiples of 8", K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N, "qkv_rope_skinny_bf16: leading dimensions too small");
   FMS_REQUIRE(head_dim % 2 == 0 && N % 16 == 0, "qkv_rope_skinny_bf16: head size %d must be even and the row a multiple of 16",
@@ -706,14 +706,14 @@ extern "C" int fmsamd_qkv_rope_skinny_bf16(const void* x, long ldx, const void* 
 //   partials[m, i] = sums of resid[m]^2 over groups of up to 16 columns, the unused ones zero
 //                    [M, partial_count], partial_count >= fmsamd_gemm_skinny_residual_partials(M, N, K)
 // A product that takes `scaled` with these partials as its deferred row norm then equals the product of the
-// normed stream.  M <= 128.
+// normed stream.  M <= 192.
 extern "C" int fmsamd_gemm_skinny_residual_partials(int M, int N, int K) {
   if (M > 16 && !skinny_takes_many_rows(M, N, K)) return ceil_div(N, 16);
   const int rows = skinny_rows_per_block(N, M);
   return ceil_div(N, rows) * (rows > 16 ? 2 : 1);
 }
 
-// Bytes of workspace that the products for at most 128 rows need (none up to 16 rows).  rows: all rows of W.
+// Bytes of workspace that the products for at most 192 rows need (none up to 16 rows).  rows: all rows of W.
 extern "C" long fmsamd_gemm_skinny_workspace(int M, int rows, int K) {
   return M > 16 && M <= FMS_SKINNY_MAX_ROWS ? wide_workspace_bytes(M, rows, K) : 0;  // enough for every product of this shape
 }
@@ -725,7 +725,7 @@ extern "C" int fmsamd_gemm_skinny_residual_bf16(const void* x, long ldx, const v
                                                 const fmsamd_row_scale* row_scale, void* workspace,
                                                 long workspace_bytes, hipStream_t stream) {
   if (M == 0 || N == 0) return 0;
-  FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 128)", M, N, K);
+  FMS_REQUIRE(M > 0 && M <= FMS_SKINNY_MAX_ROWS && N > 0 && K > 0, "gemm_skinny_residual_bf16: bad sizes M=%d N=%d K=%d (M <= 192)", M, N, K);
   FMS_REQUIRE(K % 8 == 0 && ldx % 8 == 0, "gemm_skinny_residual_bf16: K=%d and the row stride %ld must be multiples of 8",
               K, ldx);
   FMS_REQUIRE(ldx >= K && ldo >= N && ldr >= N, "gemm_skinny_residual_bf16: leading dimensions too small");

@@ -1,4 +1,4 @@
-// What the bfloat16 products for few rows (gemm.hip: at most 16 rows; gemm_wide.hip: 17 to 128) do with a
+// What the bfloat16 products for few rows (gemm.hip: at most 16 rows; gemm_wide.hip: 17 to 192) do with a
 // finished output element, and the arguments of those epilogues.
 #pragma once
 
@@ -50,9 +50,9 @@ struct RopeEpilogue {
 };
 
 
-#define FMS_SKINNY_MAX_ROWS 128
+#define FMS_SKINNY_MAX_ROWS 192
 
-// ---- 17 to 128 rows (gemm_wide.hip) ------------------------------------------
+// ---- 17 to 192 rows (gemm_wide.hip) ------------------------------------------
 // The product runs as two kernels: blocks of 128 weight rows times a slice of K leave float32 partial sums
 // in a workspace [slices][M][rows]; a second kernel adds the slices in a fixed order and applies the epilogue.
 // `rows` counts all rows of W (for the gated product both halves).

@@ -1,4 +1,4 @@
-// bfloat16 products y = x W^T for 17 to 128 rows of x, weights [rows, K] with K contiguous.
+// bfloat16 products y = x W^T for 17 to 192 rows of x, weights [rows, K] with K contiguous.
 //
 // With this many rows of x the activations are no longer small beside the weights: a block that owns 16
 // weight rows and all of K (gemm.hip) reads four times as many bytes of x as of W.  Here a block owns 128
@@ -8,12 +8,17 @@
 // kernel adds them in a fixed order (the same bits whatever the launch looks like) and applies the epilogue.
 // A product with enough weight rows for one slice (the gated feed-forward product, the output head) is
 // finished by the product kernel itself.
+// Above 128 rows the registers no longer hold four steps of x nor the operands of four tiles: the rows of x (which
+// come from L2, not from memory) are asked for one step ahead and multiplied two tiles at a time.  (Also built for
+// these row counts and measured slower: one buffer of x with a barrier on either side of its filling, and blocks of
+// four waves with 32 weight rows each on 32x32x16 matrix instructions, which read x from LDS half as often but
+// leave a SIMD with a single wave to hide its waits.)
 #include "gemm_epilogue.h"
 
 #define WD_ROWS 128   // weight rows per block
 #define WD_GROUP 128  // k-values per step of the stream
 #define WD_COMPUTE_UNITS 256
-#define WD_MAX_ROWS FMS_SKINNY_MAX_ROWS  // rows of x: eight tiles of 16
+#define WD_MAX_ROWS FMS_SKINNY_MAX_ROWS  // rows of x: twelve tiles of 16
 #define WD_DEPTH 4       // steps whose loads are in flight (even)
 #define WD_TILE_LD 132   // floats per row of the block's result tile in LDS: 128 and a shift of the banks
 
@@ -49,6 +54,8 @@ template <int MT, int MODE, typename OutT>
 __global__ void __launch_bounds__(512)
     wide_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, float* __restrict__ part, int M,
                 int rows, int K, int groups_per_slice, WideOut o) {
+  constexpr bool TALL = MT > 8;                          // more than 128 rows of x
+  constexpr int XDEPTH = TALL ? 2 : WD_DEPTH;            // steps whose loads of x are in flight: the registers hold no more
   constexpr int XS_BYTES = 2 * MT * 16 * WD_GROUP * 2;  // two steps of x: one read, one written
   constexpr int WS_BYTES = 8 * 16 * WD_GROUP * 2;       // a weight tile per wave
   constexpr int TILE_BYTES = MT * 16 * WD_TILE_LD * 4;  // the block's results, once the stream has ended
@@ -122,23 +129,25 @@ __global__ void __launch_bounds__(512)
   // The blocks walk their slice from different starting steps and wrap around: blocks that all read the same
   // 256 bytes of their rows at the same time (rows lie a multiple of kilobytes apart) crowd into few memory
   // channels.  The start depends on the block's place only, so the order of the sum does too.
-  bf16x8 xr[WD_DEPTH][XP], wr[WD_DEPTH][4];
+  bf16x8 xr[XDEPTH][XP], wr[WD_DEPTH][4];
   const int n_steps = g_end - g_begin;
   const int rot = (blockIdx.x * 5) % n_steps;
   auto group_of = [&](int t) {  // the k-group of the slice's step t (steps past the end repeat the last one)
     const int u = (t < n_steps ? t : n_steps - 1) + rot;
     return g_begin + (u >= n_steps ? u - n_steps : u);
   };
+  // (a step asks for its rows of x before its rows of W: loads come back in the order they were asked for, and with
+  // many rows of x those are asked for one step ahead only; they come from L2, not from memory)
 #pragma unroll
   for (int d = 0; d < WD_DEPTH - 1; ++d) {
-    load_x(group_of(d), xr[d]);
+    if (d < XDEPTH - 1) load_x(group_of(d), xr[d]);
     load_w(group_of(d), wr[d]);
   }
   if (MODE != WD_PARTIAL) {
     // 1 / rms of the rows of x, if their norm was left to this product.  The partial sums are asked for behind the
     // stream's first loads and all at once: in front of them, one round trip after the other, they kept the
     // stream from starting for as long as four of its steps take.
-    constexpr int RPW = MT * 2, PRE = 4;  // rows a wave, loads a row that are under way together (256 sums)
+    constexpr int RPW = MT * 2, PRE = TALL ? 2 : 4;  // rows a wave, loads a row that are under way together
     if (o.scale.partials != nullptr) {
       float pre[RPW][PRE];
 #pragma unroll
@@ -166,12 +175,12 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int d = 0; d < WD_DEPTH; ++d) {
       const int cur = t + d;
-      constexpr int ahead = WD_DEPTH - 1;
-      load_x(group_of(cur + ahead), xr[(d + ahead) % WD_DEPTH]);
+      constexpr int ahead = WD_DEPTH - 1, x_ahead = XDEPTH - 1;
+      load_x(group_of(cur + x_ahead), xr[(d + x_ahead) % XDEPTH]);
       load_w(group_of(cur + ahead), wr[(d + ahead) % WD_DEPTH]);
       const int buf = d & 1;  // WD_DEPTH is even: steps alternate between the two x buffers
       const int cur_g = group_of(cur);
-      store_x(cur_g, buf, xr[d]);
+      store_x(cur_g, buf, xr[d % XDEPTH]);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = 4 * q + lrow;
@@ -185,9 +194,9 @@ __global__ void __launch_bounds__(512)
           a[st] = *reinterpret_cast<const bf16x8*>(ws + r * WD_GROUP + (((st * 4 + g) ^ r) & 15) * 8);
         // all operands of four tiles of x first, then their products: a read that waits in front of every
         // product would pay the LDS latency sixteen times a step
+        constexpr int JT = TALL ? 2 : (MT < 4 ? MT : 4);  // many rows: the registers hold the operands of two tiles
 #pragma unroll
-        for (int j0 = 0; j0 < MT; j0 += 4) {
-          constexpr int JT = MT < 4 ? MT : 4;
+        for (int j0 = 0; j0 < MT; j0 += JT) {
           bf16x8 b[JT][4];
 #pragma unroll
           for (int jj = 0; jj < JT; ++jj)
@@ -479,8 +488,12 @@ static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float
     FMS_WK(6);
   else if (mt == 7)
     FMS_WK(7);
-  else
+  else if (mt == 8)
     FMS_WK(8);
+  else if (mt <= 10)  // many rows: tiles in pairs (their operands are taken two at a time); an empty tile is zeros
+    FMS_WK(10);
+  else
+    FMS_WK(12);
 #undef FMS_WK
 }
 

@@ -237,7 +237,7 @@ def qkv_rope_write(
     head_dim: int,
     row_norm: Optional[RowNorm] = None,
 ) -> torch.Tensor:
-    """The fused qkv projection of a decode step (at most 128 rows, bfloat16): x W^T (+ bias), q and k
+    """The fused qkv projection of a decode step (at most QKV_ROPE_MAX_ROWS rows, bfloat16): x W^T (+ bias), q and k
     rotated, k and v written into their cache pages.  Returns the [M, (H+2K)*D] buffer whose query
     columns hold the rotated queries (its other columns are not written).  Equal to `linear` followed
     by `rope_kv_write`."""
@@ -271,7 +271,7 @@ def qkv_rope_write(
     return out
 
 
-QKV_ROPE_MAX_ROWS = 128
+QKV_ROPE_MAX_ROWS = 192
 
 
 def rope_kv_write(
@@ -432,10 +432,10 @@ def prefill_qblock(nheads: int, kvheads: int, head_dim: int, n_tokens: int) -> i
 # --------------------------------------------------------------------------
 # matrix products
 # --------------------------------------------------------------------------
-SKINNY_MAX_ROWS = 128
+SKINNY_MAX_ROWS = 192
 # Up to this many rows the skinny kernel, with the norms, rotation and activation fused into it, beats the
 # vendor library followed by those as kernels of their own.
-SKINNY_FAST_ROWS = 128
+SKINNY_FAST_ROWS = 192
 
 
 def linear(
@@ -449,7 +449,7 @@ def linear(
     """x [M, K] @ weight[N, K]^T (+ bias) -> [M, N].
 
     float32 x float32: the FMA kernel (true 32-bit).  bfloat16 x bfloat16: the weight-streaming
-    skinny kernels up to 128 rows; above that the vendor library (hipBLASLt through torch.matmul,
+    skinny kernels up to 192 rows; above that the vendor library (hipBLASLt through torch.matmul,
     as the reference's nn.Linear does) for bfloat16 output, or this package's MFMA kernels when
     float32 output is wanted or allow_library is False.
     A float32 weight with bfloat16 activations (a tensor the checkpoint keeps in 32-bit) runs the
@@ -468,7 +468,7 @@ def linear(
     out_dtype = out_dtype or x.dtype
     lib = load()
     if row_norm is not None and not (weight.dtype == x.dtype == torch.bfloat16 and M <= SKINNY_FAST_ROWS):
-        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 128 rows")
+        raise ValueError(f"a deferred row norm goes with the bfloat16 product of at most {SKINNY_FAST_ROWS} rows")
     if weight.dtype == torch.float32:
         xf = x if x.dtype == torch.float32 else cast(x.contiguous(), torch.float32)
         bf = bias if bias is None or bias.dtype == torch.float32 else cast(bias, torch.float32)
@@ -520,7 +520,7 @@ def linear_into_stream(
     eps: float,
     row_norm: Optional[RowNorm] = None,
 ):
-    """The last product of a residual branch with what follows it (bfloat16, at most 128 rows):
+    """The last product of a residual branch with what follows it (bfloat16, at most SKINNY_FAST_ROWS rows):
     resid += x W^T (+ bias) in float32 in place.  Returns (scaled, RowNorm): scaled = resid * norm_weight in
     bfloat16 and the sums of squares of resid's rows by tiles of 16 columns, which a product takes as its
     `row_norm` to read the RMS-normed stream without a norm kernel in between."""
@@ -578,7 +578,7 @@ def gated_linear(
                                                    _row_scale(row_norm, M), _ptr(ws), ws_bytes, _stream()))
         return out
     if row_norm is not None:
-        raise ValueError("a deferred row norm goes with the bfloat16 product of at most 128 rows")
+        raise ValueError(f"a deferred row norm goes with the bfloat16 product of at most {SKINNY_FAST_ROWS} rows")
     gu = linear(x, weight, None, allow_library=allow_library)
     return gated_act(gu, bias, activation)
 

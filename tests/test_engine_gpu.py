@@ -665,8 +665,8 @@ def varied_lengths(n, longest):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", sorted(CONFIGS))
 def test_decode_batches_of_many_sequences(lib, folders, name, dtype):
-    """Decode steps of 20, 48, 70, 128 and 140 sequences of unequal lengths (the products for 17 to 128 rows, their
-    row buckets with padding rows, and the step above 128 rows), through captured graphs and as eager steps:
+    """Decode steps of 20, 48, 70, 128, 140 and 200 sequences of unequal lengths (the products for 17 to 192 rows, their
+    row buckets with padding rows, and the step above 192 rows), through captured graphs and as eager steps:
     both follow the plain implementation.  After three steps every third
     sequence ends and the batch goes on smaller."""
     from fms_amd.engine import Engine
@@ -675,7 +675,7 @@ def test_decode_batches_of_many_sequences(lib, folders, name, dtype):
     cfg, weights = plain(folders, name)
     model = get(lib, folders, name, dtype)
     greedy = SamplingParams(do_sample=False)
-    for n_seqs in (20, 48, 70, 128, 140):
+    for n_seqs in (20, 48, 70, 128, 140, 200):
         lens = varied_lengths(n_seqs, 130)
         room = sum(-(-(n + 8) // 64) * 64 for n in lens)
         replayed = Engine(model, max_tokens=room, max_slots=n_seqs, use_graphs=True)

@@ -187,7 +187,7 @@ def test_rope_kv_write(ops, dtype, H, K, D, rot, starts, lens):
             assert float(kc[p].abs().sum()) == 0 and float(vc[p].abs().sum()) == 0
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 32, 40, 64, 81, 128])
+@pytest.mark.parametrize("M", [1, 8, 20, 32, 40, 64, 81, 128, 129, 150, 161, 192])
 @pytest.mark.parametrize("H,K,D,rot,E", [(4, 2, 16, 16, 64), (3, 1, 48, 48, 40), (8, 8, 32, 16, 256), (40, 4, 128, 128, 32), (30, 2, 136, 136, 32)])
 def test_qkv_rope_write_equals_the_separate_kernels(ops, M, H, K, D, rot, E):
     """The decode-time fusion (projection + rotation + cache write) against linear followed by rope_kv_write."""
@@ -452,7 +452,7 @@ def test_gemm_f32(ops, M, N, K):
     torch.testing.assert_close(out, (x.double() @ w.double().t() + b.double()).float(), atol=1e-4, rtol=1e-5)
 
 
-@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 48, 64, 65, 96, 100, 128, 129, 300])
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 33, 48, 64, 65, 96, 100, 128, 129, 144, 160, 170, 192, 193, 300])
 @pytest.mark.parametrize("N,K", [(40, 24), (100, 176), (257, 96), (384, 96), (4096 + 16, 512), (20000, 64)])
 def test_gemm_bf16(ops, M, N, K):
     torch.manual_seed(7)
@@ -502,7 +502,7 @@ def test_gemm_bf16_of_widths_that_are_no_multiple_of_8(ops, M, N, K):
         torch.testing.assert_close(out, want, atol=4e-2, rtol=2e-2)
 
 
-@pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100, 128, 150])
+@pytest.mark.parametrize("M", [1, 8, 20, 40, 64, 100, 128, 130, 150, 177, 192, 200])
 @pytest.mark.parametrize("hidden,K", [(44, 24), (77, 40), (176, 64), (1000, 96)])
 def test_gated_linear(ops, M, hidden, K):
     torch.manual_seed(8)
@@ -517,7 +517,7 @@ def test_gated_linear(ops, M, hidden, K):
             torch.testing.assert_close(out, want, **(dict(atol=1e-4, rtol=1e-4) if dtype == torch.float32 else dict(atol=4e-2, rtol=2e-2)))
 
 
-@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 64, 90, 128])
+@pytest.mark.parametrize("M", [1, 7, 16, 17, 32, 33, 64, 90, 128, 140, 165, 192])
 @pytest.mark.parametrize("N,K,eps", [(48, 24, 1e-5), (96, 176, 1e-6), (4096 + 40, 64, 1e-5), (100, 96, 1e-3), (6144, 32, 1e-5)])
 def test_linear_into_stream_and_deferred_row_norm(ops, M, N, K, eps):
     """The last product of a branch adds to the float32 stream and leaves the next norm's input; the
@@ -568,7 +568,7 @@ def test_decode_products_at_the_layer_sizes_of_other_variants(ops, E, F, H, K):
     """The four products of a layer as a decode step runs them, at the sizes of the 13B, 70B and granite 3B variants
     (the 8B and 7B sizes run through whole models in test_model_shapes_gpu.py): output projection into the stream,
     gate/up with the activation and the deferred norm, down projection into the stream, qkv with rotation and cache
-    write and the deferred norm.  Row counts of the kernels for up to 16 rows, for 17 to 32 and for 33 to 128.
+    write and the deferred norm.  Row counts of the kernels for up to 16 rows, for 17 to 32, for 33 to 128 and for 129 to 192.
     References are float32 products of the same operands, on the GPU."""
     torch.manual_seed(31)
     D = E // H
@@ -579,7 +579,7 @@ def test_decode_products_at_the_layer_sizes_of_other_variants(ops, E, F, H, K):
     wqkv = (torch.randn((H + 2 * K) * D, E, device="cuda") * 0.02).bfloat16()
     nw = (1 + 0.1 * torch.randn(E, device="cuda")).bfloat16()
     cos, sin = ops.rope_table(dev(P.rope_frequencies(D, 10000.0)), 512)
-    for M in (8, 24, 80):
+    for M in (8, 24, 80, 150):
         attn = torch.randn(M, E, device="cuda").bfloat16()
         resid = torch.randn(M, E, device="cuda") * 2
         resid[0] *= 20
@@ -649,13 +649,13 @@ def test_qkv_rope_write_takes_a_deferred_row_norm(ops):
 @pytest.mark.parametrize("vocab,width", [(128256, 4096), (32000, 4096), (49152, 2560)])
 def test_output_head_at_served_vocabularies(ops, vocab, width):
     """The last product of a step at the vocabularies and widths of the registered variants: float32 logits from
-    bfloat16 rows, for the row counts of decode batches (the weight-streaming kernels, 1 to 128 rows, in blocks of
+    bfloat16 rows, for the row counts of decode batches (the weight-streaming kernels, 1 to 192 rows, in blocks of
     thousands) and above (this package's MFMA kernel), against the float32 product of the same operands; and the
     token choice on those logits."""
     torch.manual_seed(21)
     w = (torch.randn(vocab, width, device="cuda") * 0.02).bfloat16()
     wf = w.float()
-    for M in (1, 8, 17, 33, 64, 128, 130):
+    for M in (1, 8, 17, 33, 64, 128, 130, 192, 200):
         x = torch.randn(M, width, device="cuda").bfloat16()
         got = ops.linear(x, w, None, out_dtype=torch.float32)
         want = x.float() @ wf.t()

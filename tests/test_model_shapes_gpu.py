@@ -2,8 +2,8 @@
 heads) and of the Llama-2-7B shape (as many kv heads as heads), with a vocabulary cut to 4096 so that the plain
 implementation on the CPU stays cheap.  These sizes take other kernels than the tiny configurations do: the
 prefill attention with its head size known at compile time, the decode attention that stages pages in LDS, the
-weight-streaming products with thousands of columns and their variants for 17 to 128 rows, vendor products above
-128 rows.  float32 and bfloat16 against the plain implementation, and bfloat16 against the engine's own float32
+weight-streaming products with thousands of columns and their variants for 17 to 192 rows, vendor products above
+192 rows.  float32 and bfloat16 against the plain implementation, and bfloat16 against the engine's own float32
 path: whole prompts, the last 32 tokens one by one, ragged batches with reused slots, and decode batches of 5
 to 140 sequences through captured graphs.  A third model has the depth of the served ones (32 layers) at a narrower
 width.
@@ -166,9 +166,9 @@ def prompt_lengths(n):
     return [(special[i] if i < len(special) else 2 + (53 * i * i + 17 * i) % 250) for i in range(n)]
 
 
-@pytest.mark.parametrize("n_seqs", [5, 24, 64, 80, 128, 140])
+@pytest.mark.parametrize("n_seqs", [5, 24, 64, 80, 128, 140, 180])
 def test_decode_batches_through_graphs(shape, n_seqs):
-    """bfloat16 decode steps of 5 to 140 sequences of unequal lengths (above 128 the products are the vendor's
+    """bfloat16 decode steps of 5 to 180 sequences of unequal lengths (above 192 rows, which the tiny configurations run, the products are the vendor's
     and nothing is fused), as generation runs them
     (decode_and_choose: a captured graph, the token choice inside it), against the engine's float32 path fed
     the same tokens, and both against the plain implementation.  After three steps every third sequence ends."""
@@ -230,7 +230,7 @@ def test_decode_batches_through_graphs(shape, n_seqs):
 
 
 def test_replayed_and_eager_steps_choose_the_same_tokens(shape):
-    """At these sizes too (the products for 17 to 128 rows cut K by the number of rows, the decode attention splits
+    """At these sizes too (the products for 17 to 192 rows cut K by the number of rows, the decode attention splits
     by it): an eager decode step is filled up to the rows of the captured step, so generation through graphs and
     through eager steps gives the same tokens bit for bit while the batch shrinks through the row buckets."""
     from fms_amd.engine import Engine
