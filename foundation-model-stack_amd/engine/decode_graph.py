@@ -25,7 +25,7 @@ from ..cache import pages_for
 from ..kernels import ops
 from .batch import StepBatch
 
-ROW_BUCKETS = (1, 2, 4, 8, 12, 16, 20, 24, 32, 40, 48, 56, 64, 80, 96, 112, 128, 192, 256)
+ROW_BUCKETS = (1, 2, 4, 8, 12, 16, 20, 24, 32, 40, 48, 56, 64, 80, 96, 112, 128, 160, 192, 256)
 CONTEXT_BUCKET = 2048  # the smallest context bound of a graph; larger ones double
 CONTEXT_HEADROOM = 256  # a new graph is captured for a bound this far beyond the longest context
 
