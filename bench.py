@@ -6,7 +6,7 @@ Random weights, synthetic token ids.  A "step" is one decode step of the whole b
 the library's own generation path (step function, cache, kernels, sampler).  One JSON line is
 printed: decode tokens/s at batch 8 (`value`), the prefill of 2,048 tokens, the decode step's
 memory roofline (against the published peak and against what a pure read reaches on this GPU now),
-the share of the step's time by kernel class, and further points: decode at batch 1 and 64, at
+the share of the step's time by kernel class, and further points: decode at batch 1, 64 and 192, at
 batch 8 with every context near 8000 tokens, the Llama-2-7B shape at batch 8 (256 steps) and the
 Llama-3-70B shape at batch 16 (128 steps).  Decode steps run as generation runs them: the host looks
 at the chosen tokens every `steps_ahead` steps (`--steps-ahead 1`: after every step).
@@ -217,7 +217,7 @@ def main() -> int:
         points[f"{name}_frac"] = round(gbs / HBM_GBS, 4)
 
     if not args.skip_points and args.only is None:
-        for b, steps, warmup in ((1, min(args.steps, 32), 4), (64, min(args.steps, 16), 2)):
+        for b, steps, warmup in ((1, min(args.steps, 32), 4), (64, min(args.steps, 16), 2), (192, min(args.steps, 12), 2)):
             point(f"decode_b{b}", *decode(b, steps, warmup))
         # every context near the benchmark's context length
         near = min(8000, args.context - 64)
