@@ -9,11 +9,10 @@ no padding: tokens of all sequences are laid end to end.
 
 from __future__ import annotations
 
-from typing import List, Optional, Sequence, Union  # noqa: F401
+import os
+from typing import List, Optional, Sequence, Union
 
 import torch
-
-import os
 
 from ..cache import pages_for
 from ..sampling import SamplingParams, choose
