@@ -72,7 +72,7 @@ __global__ void __launch_bounds__(512)
   int n0 = blockIdx.x * WD_ROWS + wave * 16, n_end = rows;
   if (MODE == WD_GATED) {
     const int first = blockIdx.x * o.gate_rows + (wave & 3) * 16;
-    const int last = (blockIdx.x + 1) * o.gate_rows < o.N ? (blockIdx.x + 1) * o.gate_rows : o.N;  // the block's end
+    const int last = ((int)blockIdx.x + 1) * o.gate_rows < o.N ? ((int)blockIdx.x + 1) * o.gate_rows : o.N;  // the block's end
     n0 = wave < 4 ? first : o.tile2_offset + first;
     n_end = wave < 4 ? last : o.tile2_offset + last;
   }
@@ -229,7 +229,7 @@ __global__ void __launch_bounds__(512)
     // 16 threads a row: four gate columns and their four up columns each
     const int c = 4 * (threadIdx.x & 15);
     const int n = blockIdx.x * o.gate_rows + c;
-    const int n_hi = (blockIdx.x + 1) * o.gate_rows < o.N ? (blockIdx.x + 1) * o.gate_rows : o.N;
+    const int n_hi = ((int)blockIdx.x + 1) * o.gate_rows < o.N ? ((int)blockIdx.x + 1) * o.gate_rows : o.N;
     OutT* const out = (OutT*)o.out;
 #pragma unroll
     for (int p = 0; p < (MT + 1) / 2; ++p) {
