@@ -8,6 +8,10 @@
 // kernel adds them in a fixed order (the same bits whatever the launch looks like) and applies the epilogue.
 // A product with enough weight rows for one slice (the gated feed-forward product, the output head) is
 // finished by the product kernel itself.
+// From 33 to 128 rows the products are 32x32x16 matrix instructions on tiles of 32 weight rows and 32 rows of x, two
+// waves to a tile row (a kernel of nothing but those instructions runs at twice the rate of one of 16x16x32 on this
+// GPU, and a wave then reads half the rows of x from LDS): 9.66 against 9.97 ms a decode step of 128 sequences of the
+// Llama-3-8B shape, 8.14 against 8.36 of 96, 6.29 against 6.32 of 64.
 // Above 128 rows the registers no longer hold four steps of x nor the operands of four tiles: the rows of x (which
 // come from L2, not from memory) are asked for one step ahead and multiplied two tiles at a time.  (Also built for
 // these row counts and measured slower: one buffer of x with a barrier on either side of its filling, and blocks of
@@ -50,16 +54,23 @@ __device__ __forceinline__ void store4(bf16* p, f32x4 v) {
 // Loads are 16 rows' 256 contiguous bytes as 4 instructions of 4 rows (what the memory system streams at
 // full rate); LDS holds them as loaded, with the 16-byte pieces of a row XOR-swizzled by the row, and gives
 // them back in the MFMA operand layout (lane (r, g) takes row r, k-step s at piece 4 s + g).
-template <int MT, int MODE, typename OutT>
+template <int MT, int MODE, typename OutT, bool SQ>
 __global__ void __launch_bounds__(512)
     wide_kernel(const bf16* __restrict__ x, long ldx, const bf16* __restrict__ w, float* __restrict__ part, int M,
                 int rows, int K, int groups_per_slice, WideOut o) {
   constexpr bool TALL = MT > 8;                          // more than 128 rows of x
   constexpr int XDEPTH = TALL ? 2 : WD_DEPTH;            // steps whose loads of x are in flight: the registers hold no more
-  constexpr int XS_BYTES = 2 * MT * 16 * WD_GROUP * 2;  // two steps of x: one read, one written
-  constexpr int WS_BYTES = 8 * 16 * WD_GROUP * 2;       // a weight tile per wave
-  constexpr int TILE_BYTES = MT * 16 * WD_TILE_LD * 4;  // the block's results, once the stream has ended
-  constexpr int SMEM = XS_BYTES + WS_BYTES > TILE_BYTES ? XS_BYTES + WS_BYTES : TILE_BYTES;
+  // SQ: products of 32 weight rows against 32 rows of x (32x32x16; a kernel of nothing but those runs at twice the rate
+  // of one of 16x16x32 products on this GPU).  The waves form four rows of two: a pair shares 32 weight rows (each
+  // wave loads 16 of them) and deals the tiles of 32 rows of x between its two waves, so that a wave reads half the
+  // rows of x from LDS.  The weight tiles are then read by a neighbour too, and have two buffers like x.
+  constexpr int MT32 = (MT + 1) / 2;                     // SQ: tiles of 32 rows of x
+  constexpr int XROWS = SQ ? MT32 * 32 : MT * 16;        // rows of x in LDS
+  constexpr int WBUFS = SQ ? 2 : 1;
+  constexpr int XS_BYTES = 2 * XROWS * WD_GROUP * 2;     // two steps of x: one read, one written
+  constexpr int WS_BYTES = 8 * 16 * WD_GROUP * 2;        // a weight tile per wave
+  constexpr int TILE_BYTES = XROWS * WD_TILE_LD * 4;     // the block's results, once the stream has ended
+  constexpr int SMEM = XS_BYTES + WBUFS * WS_BYTES > TILE_BYTES ? XS_BYTES + WBUFS * WS_BYTES : TILE_BYTES;
   __shared__ __attribute__((aligned(16))) char smem[SMEM];
   __shared__ float row_scale[MT * 16];
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
@@ -68,6 +79,8 @@ __global__ void __launch_bounds__(512)
   float* const tile = reinterpret_cast<float*>(smem);
   const int r = lane & 15, g = lane >> 4;
   const int lrow = lane >> 4, seg = lane & 15;
+  const int li = lane & 31, kb = lane >> 5;     // SQ: the lane's row of a 32-row tile and its half of a k-step's 16 values
+  const int pair = wave >> 1, side = wave & 1;  // SQ: the wave's row of waves, and which of its two waves it is
   // the wave's 16 weight rows start at n0; rows from n_end on are not the wave's to read
   int n0 = blockIdx.x * WD_ROWS + wave * 16, n_end = rows;
   if (MODE == WD_GATED) {
@@ -85,10 +98,10 @@ __global__ void __launch_bounds__(512)
   // Loads never sit behind a branch and their data is not touched before the step that uses it (either makes
   // the compiler wait for every load in flight): a piece out of range is read from a valid address, and is
   // replaced by zeros only when it goes to LDS.
-  constexpr int XP = (MT * 256 + 511) / 512;
+  constexpr int XP = (XROWS * 16 + 511) / 512;
   auto x_ok = [&](int grp, int i) {
     const int id = threadIdx.x + i * 512;
-    return id < MT * 256 && (id >> 4) < M && grp * WD_GROUP + (id & 15) * 8 < K;
+    return id < XROWS * 16 && (id >> 4) < M && grp * WD_GROUP + (id & 15) * 8 < K;
   };
   auto w_ok = [&](int grp, int q) { return n0 + 4 * q + lrow < n_end && grp * WD_GROUP + seg * 8 < K; };
   auto load_x = [&](int grp, bf16x8 (&xr)[XP]) {
@@ -104,8 +117,8 @@ __global__ void __launch_bounds__(512)
     for (int i = 0; i < XP; ++i) {
       const int id = threadIdx.x + i * 512;
       const int m = id >> 4, piece = id & 15;
-      if (id < MT * 256)
-        *reinterpret_cast<bf16x8*>(xs + buf * (MT * 16 * WD_GROUP) + m * WD_GROUP + ((piece ^ m) & 15) * 8) =
+      if (id < XROWS * 16)
+        *reinterpret_cast<bf16x8*>(xs + buf * (XROWS * WD_GROUP) + m * WD_GROUP + ((piece ^ m) & 15) * 8) =
             x_ok(grp, i) ? xr[i] : zero;
     }
   };
@@ -117,9 +130,15 @@ __global__ void __launch_bounds__(512)
     }
   };
 
-  f32x4 acc[MT];
+  f32x4 acc[SQ ? 1 : MT];
 #pragma unroll
-  for (int j = 0; j < MT; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < (SQ ? 1 : MT); ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+  constexpr int NT32 = (MT32 + 1) / 2;  // SQ: tiles of x a wave takes at most (tiles side, side + 2, ...)
+  f32x16 acc32[SQ ? NT32 : 1];
+#pragma unroll
+  for (int j = 0; j < (SQ ? NT32 : 1); ++j)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) acc32[j][v] = 0.f;
 
   // WD_DEPTH steps in flight: while step t multiplies, the loads of steps t + 1 .. t + WD_DEPTH - 1 are under
   // way (a load takes several steps' time to arrive).  Every step issues the loads of the step WD_DEPTH - 1
@@ -181,13 +200,37 @@ __global__ void __launch_bounds__(512)
       const int buf = d & 1;  // WD_DEPTH is even: steps alternate between the two x buffers
       const int cur_g = group_of(cur);
       store_x(cur_g, buf, xr[d % XDEPTH]);
+      bf16* const wsb = ws + (SQ ? buf * (WS_BYTES / 2) : 0);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = 4 * q + lrow;
-        *reinterpret_cast<bf16x8*>(ws + row * WD_GROUP + ((seg ^ row) & 15) * 8) = w_ok(cur_g, q) ? wr[d][q] : zero;
+        *reinterpret_cast<bf16x8*>(wsb + row * WD_GROUP + ((seg ^ row) & 15) * 8) = w_ok(cur_g, q) ? wr[d][q] : zero;
       }
       block_sync_lds();  // the step's x is whole; the buffer written now was last read two steps ago
-      if (cur < n_steps) {  // uniform; a step past the end multiplies nothing
+      if (SQ) {
+        if (cur < n_steps) {  // uniform; a step past the end multiplies nothing
+          // the pair's 32 weight rows: this wave's 16 and its neighbour's, side by side in LDS
+          const bf16* const wpair = reinterpret_cast<const bf16*>(smem + XS_BYTES) + buf * (WS_BYTES / 2) + pair * 32 * WD_GROUP;
+          bf16x8 a[8];
+#pragma unroll
+          for (int st = 0; st < 8; ++st)
+            a[st] = *reinterpret_cast<const bf16x8*>(wpair + li * WD_GROUP + (((st * 2 + kb) ^ li) & 15) * 8);
+#pragma unroll
+          for (int t32 = 0; t32 < NT32; ++t32) {
+            const int jt = side + 2 * t32;  // uniform over the wave
+            if (jt < MT32) {
+              bf16x8 b[8];
+              const int m = jt * 32 + li;
+#pragma unroll
+              for (int st = 0; st < 8; ++st)
+                b[st] = *reinterpret_cast<const bf16x8*>(xs + buf * (XROWS * WD_GROUP) + m * WD_GROUP + (((st * 2 + kb) ^ m) & 15) * 8);
+#pragma unroll
+              for (int st = 0; st < 8; ++st)
+                acc32[t32] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[st], b[st], acc32[t32], 0, 0, 0);
+            }
+          }
+        }
+      } else if (cur < n_steps) {  // uniform; a step past the end multiplies nothing
         bf16x8 a[4];
 #pragma unroll
         for (int st = 0; st < 4; ++st)
@@ -221,8 +264,21 @@ __global__ void __launch_bounds__(512)
   // weight rows in the order of the waves; from there they leave in whole rows of 256 or 512 bytes.
   // acc[j][e]: the wave's weight row 4 g + e, x row 16 j + r.
   __syncthreads();
+  if (SQ) {
+    // acc32[t][v]: x row 32 (side + 2 t) + li, the pair's weight row 8 (v / 4) + 4 kb + v % 4
 #pragma unroll
-  for (int j = 0; j < MT; ++j) *reinterpret_cast<f32x4*>(tile + (j * 16 + r) * WD_TILE_LD + wave * 16 + 4 * g) = acc[j];
+    for (int t32 = 0; t32 < NT32; ++t32) {
+      const int jt = side + 2 * t32;
+      if (jt < MT32)
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+          *reinterpret_cast<f32x4*>(tile + (jt * 32 + li) * WD_TILE_LD + pair * 32 + 8 * u + 4 * kb) =
+              f32x4{acc32[t32][4 * u], acc32[t32][4 * u + 1], acc32[t32][4 * u + 2], acc32[t32][4 * u + 3]};
+    }
+  } else {
+#pragma unroll
+    for (int j = 0; j < MT; ++j) *reinterpret_cast<f32x4*>(tile + (j * 16 + r) * WD_TILE_LD + wave * 16 + 4 * g) = acc[j];
+  }
   __syncthreads();
 
   if (MODE == WD_GATED) {
@@ -474,8 +530,10 @@ template <int MODE, typename OutT>
 static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float* part, int M, int rows, int K,
                         int per_slice, const WideOut& o, hipStream_t stream) {
   const int mt = ceil_div(M, 16);
+  // 33 to 128 rows: products of 32 x 32 tiles; fewer rows are one tile of 16 or two, more than 128 do not leave room
+  // for two buffers of the weights
 #define FMS_WK(MT) \
-  wide_kernel<MT, MODE, OutT><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice, o)
+  wide_kernel<MT, MODE, OutT, (MT >= 3 && MT <= 8)><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice, o)
   if (mt == 2)
     FMS_WK(2);
   else if (mt == 3)
