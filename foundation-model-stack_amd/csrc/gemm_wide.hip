@@ -8,15 +8,14 @@
 // kernel adds them in a fixed order (the same bits whatever the launch looks like) and applies the epilogue.
 // A product with enough weight rows for one slice (the gated feed-forward product, the output head) is
 // finished by the product kernel itself.
-// From 33 to 128 rows the products are 32x32x16 matrix instructions on tiles of 32 weight rows and 32 rows of x, two
+// From 33 rows on the products are 32x32x16 matrix instructions on tiles of 32 weight rows and 32 rows of x, two
 // waves to a tile row (a kernel of nothing but those instructions runs at twice the rate of one of 16x16x32 on this
-// GPU, and a wave then reads half the rows of x from LDS): 9.66 against 9.97 ms a decode step of 128 sequences of the
-// Llama-3-8B shape, 8.14 against 8.36 of 96, 6.29 against 6.32 of 64.
-// Above 128 rows the registers no longer hold four steps of x nor the operands of four tiles: the rows of x (which
-// come from L2, not from memory) are asked for one step ahead and multiplied two tiles at a time.  (Also built for
-// these row counts and measured slower: one buffer of x with a barrier on either side of its filling, and blocks of
-// four waves with 32 weight rows each on 32x32x16 matrix instructions, which read x from LDS half as often but
-// leave a SIMD with a single wave to hide its waits.)
+// GPU, and a wave then reads half the rows of x from LDS): 9.5 against 9.97 ms a decode step of 128 sequences of the
+// Llama-3-8B shape, 8.14 against 8.36 of 96, 13.1 against 13.9 of 192.
+// Above 128 rows the registers no longer hold four steps of x: the rows of x (which come from L2, not from memory)
+// are asked for one step ahead.  (Also built for these row counts and measured slower: one buffer of x with a barrier
+// on either side of its filling, and blocks of four waves with 32 weight rows each, which leave a SIMD with a single
+// wave to hide its waits.)
 #include "gemm_epilogue.h"
 
 #define WD_ROWS 128   // weight rows per block
@@ -70,9 +69,15 @@ __global__ void __launch_bounds__(512)
   constexpr int XS_BYTES = 2 * XROWS * WD_GROUP * 2;     // two steps of x: one read, one written
   constexpr int WS_BYTES = 8 * 16 * WD_GROUP * 2;        // a weight tile per wave
   constexpr int TILE_BYTES = XROWS * WD_TILE_LD * 4;     // the block's results, once the stream has ended
-  constexpr int SMEM = XS_BYTES + WBUFS * WS_BYTES > TILE_BYTES ? XS_BYTES + WBUFS * WS_BYTES : TILE_BYTES;
+  // The rows' scales (1 / rms, if the norm of x was left to this product) are worked out while the first loads are
+  // under way, kept one a lane, and put into LDS behind the result tile when the stream has ended: at 192 rows the
+  // stream's buffers take all of LDS.
+  constexpr int STREAM_BYTES = XS_BYTES + WBUFS * WS_BYTES;
+  constexpr int SMEM = STREAM_BYTES > TILE_BYTES + MT * 16 * 4 ? STREAM_BYTES : TILE_BYTES + MT * 16 * 4;
+  static_assert(SMEM <= 160 * 1024, "the stream's buffers must fit the LDS of a compute unit");
   __shared__ __attribute__((aligned(16))) char smem[SMEM];
-  __shared__ float row_scale[MT * 16];
+  float* const row_scale = reinterpret_cast<float*>(smem + TILE_BYTES);
+  float my_scale = 1.f;  // of row wave * RPW + lane, for lane < RPW
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1);
   bf16* const xs = reinterpret_cast<bf16*>(smem);
   bf16* const ws = reinterpret_cast<bf16*>(smem + XS_BYTES) + wave * 16 * WD_GROUP;
@@ -184,10 +189,8 @@ __global__ void __launch_bounds__(512)
         for (int j = 0; j < PRE; ++j) sum += lane + j * WAVE < o.scale.count ? pre[k][j] : 0.f;
         for (int i = lane + PRE * WAVE; i < o.scale.count; i += WAVE) sum += o.scale.partials[(size_t)m * o.scale.count + i];
         const float total = wave_sum(sum);
-        if (lane == 0) row_scale[wave * RPW + k] = rsqrtf(total * o.scale.inv_width + o.scale.eps);
+        if (lane == k) my_scale = rsqrtf(total * o.scale.inv_width + o.scale.eps);
       }
-    } else if (lane < RPW) {
-      row_scale[wave * RPW + lane] = 1.f;
     }
   }
   for (int t = 0; t < n_steps; t += WD_DEPTH) {
@@ -279,6 +282,7 @@ __global__ void __launch_bounds__(512)
 #pragma unroll
     for (int j = 0; j < MT; ++j) *reinterpret_cast<f32x4*>(tile + (j * 16 + r) * WD_TILE_LD + wave * 16 + 4 * g) = acc[j];
   }
+  if (MODE != WD_PARTIAL && lane < MT * 2) row_scale[wave * (MT * 2) + lane] = my_scale;
   __syncthreads();
 
   if (MODE == WD_GATED) {
@@ -530,10 +534,9 @@ template <int MODE, typename OutT>
 static void launch_wide(dim3 grid, const void* x, long ldx, const void* w, float* part, int M, int rows, int K,
                         int per_slice, const WideOut& o, hipStream_t stream) {
   const int mt = ceil_div(M, 16);
-  // 33 to 128 rows: products of 32 x 32 tiles; fewer rows are one tile of 16 or two, more than 128 do not leave room
-  // for two buffers of the weights
+  // from 33 rows on: products of 32 x 32 tiles; fewer rows are one tile of 16 or two
 #define FMS_WK(MT) \
-  wide_kernel<MT, MODE, OutT, (MT >= 3 && MT <= 8)><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice, o)
+  wide_kernel<MT, MODE, OutT, (MT >= 3)><<<grid, 512, 0, stream>>>((const bf16*)x, ldx, (const bf16*)w, part, M, rows, K, per_slice, o)
   if (mt == 2)
     FMS_WK(2);
   else if (mt == 3)
