@@ -450,8 +450,8 @@ def linear(
 
     float32 x float32: the FMA kernel (true 32-bit).  bfloat16 x bfloat16: the weight-streaming
     skinny kernels up to 192 rows; above that the vendor library (hipBLASLt through torch.matmul,
-    as the reference's nn.Linear does) for bfloat16 output, or this package's MFMA kernels when
-    float32 output is wanted or allow_library is False.
+    as the reference's nn.Linear does; for float32 output with the float32 sums as they are), or this
+    package's MFMA kernel when allow_library is False.
     A float32 weight with bfloat16 activations (a tensor the checkpoint keeps in 32-bit) runs the
     float32 kernel on up-cast activations.
     """
@@ -500,8 +500,13 @@ def linear(
                                           _code(out_dtype), out.stride(0), M, N, K, _row_scale(row_norm, M), _ptr(ws),
                                           ws_bytes, _stream()))
         return out
-    if allow_library and out_dtype == torch.bfloat16:
-        out = torch.matmul(x, weight.t())  # vendor library GEMM, float32 accumulation
+    if allow_library and out_dtype in (torch.bfloat16, torch.float32):
+        # vendor library GEMM, float32 accumulation; float32 results (the logits of many rows) come straight from the
+        # accumulators, without a rounding to bfloat16 in between
+        if out_dtype == torch.bfloat16:
+            out = torch.matmul(x, weight.t())
+        else:
+            out = torch.mm(x, weight.t(), out_dtype=torch.float32)
         if bias is not None:
             bias_add_(out, bias)
         return out
